@@ -4,7 +4,7 @@ CXX ?= g++
 ARCH ?= gfx950
 HIPFLAGS = --offload-arch=$(ARCH) -O3 -std=c++17 -fPIC -Wall
 CSRC = yalm_amd/csrc
-HIP_SRCS = $(CSRC)/yalm_hip.hip $(CSRC)/prefill.hip
+HIP_SRCS = $(CSRC)/shim.hip $(CSRC)/yalm_hip.hip $(CSRC)/prefill.hip $(CSRC)/seq.hip
 HIP_OBJS = $(patsubst $(CSRC)/%.hip,build/%.o,$(HIP_SRCS))
 HIP_HDRS = $(wildcard $(CSRC)/*.h) include/yalm_hip.h
 
@@ -13,11 +13,20 @@ all: yalm_amd/libyalm_hip.so oracle host
 yalm_amd/libyalm_hip.so: $(HIP_OBJS)
 	$(HIPCC) $(HIPFLAGS) -shared -o $@ $(HIP_OBJS) -L/opt/rocm/lib -lrccl -Wl,-rpath,/opt/rocm/lib
 
+# the layer-list engine alone (shim + seq): what a tool that serves only layer-list
+# models builds on demand; the same entry points are also part of libyalm_hip.so
+seq: yalm_amd/libyalm_seq.so
+yalm_amd/libyalm_seq.so: build/shim.o build/seq.o
+	$(HIPCC) $(HIPFLAGS) -shared -o $@ build/shim.o build/seq.o
+
 
 # prefill.hip: MFMA accumulators in arch VGPRs (no AGPR form): the attention kernel's O and
 # S^T accumulators are touched by VALU (softmax, rescale), and the AGPR form copied all 64 O
 # registers out and back on every key tile (260 registers -> 1 wave per SIMD; 175 without)
 build/prefill.o: HIPFLAGS += -mllvm -amdgpu-mfma-vgpr-form
+
+# the newer units are built without packed-FP32 VALU forms
+build/shim.o build/seq.o: HIPFLAGS += -Xclang -target-feature -Xclang -packed-fp32-ops
 
 build/%.o: $(CSRC)/%.hip $(HIP_HDRS)
 	@mkdir -p build
@@ -35,7 +44,7 @@ resource-usage:
 		grep -E "Function Name|VGPRs:|SGPRs|Occupancy|LDS Size" | paste - - - - - -
 
 clean:
-	rm -f yalm_amd/libyalm_hip.so $(HIP_OBJS)
+	rm -f yalm_amd/libyalm_hip.so yalm_amd/libyalm_seq.so $(HIP_OBJS)
 	$(MAKE) -C oracle clean
 	$(MAKE) -C yalm_amd/host clean
 
@@ -45,4 +54,4 @@ tools: $(addprefix tools/,$(TOOLS))
 tools/%: tools/%.hip $(HIP_HDRS)
 	$(HIPCC) --offload-arch=$(ARCH) -O3 -std=c++17 -o $@ $<
 
-.PHONY: all oracle host clean resource-usage tools
+.PHONY: all seq oracle host clean resource-usage tools

@@ -308,6 +308,95 @@ int yalm_prefill_time(yalm_decoder d, int n, int iters, float *avg_ms);
  * unknown key is YALM_ERR_ARG. */
 int yalm_set_prefill_forms(yalm_decoder d, const char *spec);
 
+/* ---------------- layer-list models: mixers and feed-forwards chosen per layer ----------------
+ * A second decoder kind beside yalm_decoder, for designs whose layers differ from one
+ * another: every layer names a token mixer (latent attention over a cached low-rank
+ * key/value latent, a real-gated linear recurrence, a gated delta rule) and a
+ * feed-forward (none, dense GLU, routed experts with an optional shared expert), each
+ * with its own sizes and constants. Around every sublayer: x += norm_b(f(norm(x))).
+ * One yalm_seq holds ONE sequence: its position, the latent caches and the recurrent
+ * and convolution states, all in HBM; yalm_seq_step appends tokens (a whole prompt, a
+ * portion of one, or a single decoded token) from where the last call stopped, so the
+ * logits do not depend on how a prompt was cut. Residual stream, norms, attention
+ * scores, routers and everything inside a recurrence are f32; weight_dtype selects the
+ * matrices: YALM_BF16 (bf16 MFMA products with f32 accumulation for portions, bf16
+ * weight-streaming GEMVs for single tokens) or YALM_F32 (true f32 products).
+ * Matrices are row-major [out][in]. */
+enum { YALM_MIX_LATENT = 0, YALM_MIX_RGLRU = 1, YALM_MIX_DELTA = 2 };
+enum { YALM_FF_NONE = 0, YALM_FF_DENSE = 1, YALM_FF_MOE = 2 };
+
+typedef struct yalm_seq_layer {
+	int mixer;                     /* YALM_MIX_* */
+	int heads, kv_heads, dim, vdim; /* latent: heads x dim queries / keys, vdim values; delta: kv_heads x dim
+	                                  queries / keys shared by heads / kv_heads value heads of vdim */
+	int kv_rank, q_rank, kv_from;  /* latent: ranks; kv_from >= 0: read that layer's latent cache (no own w_in rows) */
+	float attn_scale;              /* latent: score = q.k * attn_scale */
+	int rec_width, blocks;         /* rglru: channels, diagonal gate blocks */
+	int conv;                      /* rglru, delta: taps of the causal per-channel convolution */
+	int ff_kind, ff;               /* YALM_FF_*; ff: hidden size (dense) or one expert's (moe) */
+	int experts, top, groups, groups_keep; /* moe: top experts among the groups_keep best of `groups` groups */
+	float router_scale, limit;     /* moe: weight = softmax score * router_scale; expert clamp */
+	int shared_ff;                 /* moe: shared expert's hidden size, 0 = none */
+	float shared_limit;
+	/* f32 vectors */
+	const float *norm1, *norm1b, *norm2, *norm2b; /* [width] each; norm2* unused without a feed-forward */
+	const float *q_norm, *kv_norm;  /* latent: [q_rank], [kv_rank] */
+	const float *in_bias;           /* rglru: [2 rec_width] (gate branch, recurrent branch) */
+	const float *conv_w, *conv_b;   /* [channels][conv] (last column = current token); rglru bias [rec_width] */
+	const float *gate_a, *gate_a_b, *gate_i, *gate_i_b; /* rglru: [blocks][bs][bs], [rec_width] (bs = rec_width / blocks) */
+	const float *lam;               /* rglru: [rec_width] */
+	const float *a_log, *dt_bias, *out_norm; /* delta: [heads], [heads], [vdim] */
+	const float *router, *shared_sg; /* moe: [experts][width], [width] */
+	/* matrices of weight_dtype */
+	const void *w_in;  /* latent: [q_rank (+ kv_rank if own latent)][width] (query down, latent down);
+	                      rglru: [2 rec_width][width] (gate branch, recurrent branch);
+	                      delta: [2 kv_heads dim + 2 heads vdim + 2 heads][width] (q, k, v, output gate, beta, decay) */
+	const void *w_uq;  /* latent: [heads dim][q_rank] */
+	const void *w_ukt; /* latent: [heads][kv_rank][dim], the key up-projection transposed per head */
+	const void *w_uv;  /* latent: [heads vdim][kv_rank] */
+	const void *w_o;   /* [width][heads vdim | rec_width] */
+	const void *w_gate, *w_up, *w_down; /* dense: [ff][width] x2, [width][ff]; moe: the same per expert, stacked */
+	const void *ws_gate, *ws_up, *ws_down; /* moe shared expert */
+} yalm_seq_layer;
+
+typedef struct yalm_seq_config {
+	int width, vocab, n_layers, max_tokens; /* max_tokens: positions one sequence may hold */
+	float embed_scale, norm_eps;
+	int weight_dtype; /* YALM_BF16 | YALM_F32 */
+} yalm_seq_config;
+
+typedef struct yalm_seq_weights {
+	const void *embed;       /* [vocab][width] */
+	const float *final_norm; /* [width] */
+	const void *head;        /* [vocab][width] */
+	const yalm_seq_layer *layers; /* HOST array of n_layers entries, copied by yalm_seq_create */
+} yalm_seq_weights;
+
+typedef struct yalm_seq_s *yalm_seq;
+
+int yalm_seq_create(const yalm_seq_config *config, const yalm_seq_weights *weights, yalm_stream s, yalm_seq *out);
+int yalm_seq_destroy(yalm_seq q);
+/* The sequence ends: recurrent and convolution states zeroed, position 0 (cache rows are
+ * simply overwritten by the next sequence). */
+int yalm_seq_reset(yalm_seq q);
+int yalm_seq_pos(yalm_seq q, int *pos);
+/* Appends n tokens at the current position. want: n_want ascending indices into tokens whose
+ * logits are asked for; logits_host receives [n_want][vocab] f32 (both may be NULL / 0).
+ * Synchronous when logits are asked for. */
+int yalm_seq_step(yalm_seq q, const int *tokens, int n, const int *want, int n_want, float *logits_host);
+/* Device-resident greedy decode, as yalm_generate_greedy: feeds `token` at the current
+ * position, then n_steps - 1 more tokens, each the first-max argmax of the previous
+ * step's logits, with no host round trip per token; out_tokens gets the n_steps choices. */
+int yalm_seq_generate_greedy(yalm_seq q, int token, int n_steps, int *out_tokens);
+/* Test hook: keep the residual stream after every layer of the next steps (on = 1), and
+ * read the last step's [n_layers][n][width] f32 back. */
+int yalm_seq_layer_dump(yalm_seq q, int on);
+int yalm_seq_get_layers(yalm_seq q, float *host, size_t count);
+/* Average device time (ms) of one n-token portion at position pos0 (synthetic token ids,
+ * states left as they were found is NOT promised: call yalm_seq_reset after), over iters
+ * back-to-back runs; n = 1 times the single-token path. */
+int yalm_seq_time_step(yalm_seq q, int n, int pos0, int iters, float *avg_ms);
+
 /* ---------------- test API: replaces infer.cu:890-1019 (model.h:370-384) ---------------- */
 /* Host pointers in and out; synchronous. dtype selects the weight type
  * (matmul_cuda<float|half|uint8_t>). */

@@ -156,6 +156,19 @@ struct WF16 {
 		}
 	}
 };
+// bfloat16: the upper half of the f32 with the same value, an exact upcast.
+struct WBF16 {
+	static constexpr int EPL = 8;
+	static constexpr int BYTES = 2;
+	__device__ static __forceinline__ void unpack(const u32x4_t &w, float *o) {
+#pragma unroll
+		for (int i = 0; i < 4; ++i) {
+			const uint32_t v = w[i];
+			o[2 * i] = __builtin_bit_cast(float, v << 16);
+			o[2 * i + 1] = __builtin_bit_cast(float, v & 0xFFFF0000u);
+		}
+	}
+};
 // OCP E5M2 (== gfx950 "bf8"): the f16 with bits (b << 8), an exact upcast.
 // gfx950 converts two packed bf8 bytes to two f32 in one VALU op
 // (v_cvt_pk_f32_bf8, OCP E5M2 on CDNA4), half the work of the shift + f16

@@ -1,5 +1,6 @@
-// misc_kernels.h — per-token bookkeeping kernels: step setup + embedding row,
-// device argmax (greedy -t 0), and the deterministic synthetic initialiser.
+// misc_kernels.h — per-token bookkeeping kernels: step setup + embedding row and the
+// device argmax (greedy -t 0). Included by more than one engine unit: the non-template
+// kernels are static.
 #pragma once
 
 #include <float.h>
@@ -7,9 +8,12 @@
 #include "device_common.h"
 #include "tp_exchange.h"
 
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wunused-function" // a unit uses the kernels it needs
+
 // Host-provided (token, pos) -> device StepState. Launched eagerly ahead of a
 // graph replay; kernel arguments are captured at launch, so no host buffer race.
-__global__ void set_step_kernel(StepState *st, int token, int pos, int reset_gen) {
+static __global__ void set_step_kernel(StepState *st, int token, int pos, int reset_gen) {
 	st->token = token;
 	st->pos = pos;
 	if (reset_gen)
@@ -32,7 +36,7 @@ __device__ __forceinline__ void step_rope(StepState *st, int pos, const float *_
 
 // Explicit indices for the per-block test hook (Block::block signature); n_ex: the IPC
 // tensor-parallel exchanges the block uses (tp_exchange.h).
-__global__ void set_step_full_kernel(StepState *st, int pos, int kv_sink, int kv_pos, int kv_len, int n_ex = 0,
+static __global__ void set_step_full_kernel(StepState *st, int pos, int kv_sink, int kv_pos, int kv_len, int n_ex = 0,
                                      const float *__restrict__ inv_freq = nullptr, int half = 0) {
 	if (inv_freq)
 		step_rope(st, pos, inv_freq, half);
@@ -49,7 +53,7 @@ __global__ void set_step_full_kernel(StepState *st, int pos, int kv_sink, int kv
 
 // Timing hook (yalm_time_kernel): a new launch generation, as step_begin_kernel
 // starts one, so an in-launch hand-off never sees the previous launch's tags.
-__global__ void epoch_bump_kernel(StepState *st, int n_ex) {
+static __global__ void epoch_bump_kernel(StepState *st, int n_ex) {
 	st->epoch = st->epoch + 1u;
 	st->xbase = st->xnext;
 	st->xnext = st->xnext + (unsigned)n_ex;
@@ -59,7 +63,7 @@ __global__ void epoch_bump_kernel(StepState *st, int n_ex) {
 // 1083; KV_SINKS = 2, model.h:12) and x = embedding[token] (infer.cu:622-640);
 // n_ex: the IPC tensor-parallel exchanges this forward uses (tp_exchange.h).
 template <class WT>
-__global__ __launch_bounds__(256) void step_begin_kernel(StepState *st, const void *__restrict__ emb, int dim,
+static __global__ __launch_bounds__(256) void step_begin_kernel(StepState *st, const void *__restrict__ emb, int dim,
                                                          float *__restrict__ x, int max_seq_len, int n_ex,
                                                          const float *__restrict__ inv_freq, int half) {
 	const int token = st->token;
@@ -165,7 +169,7 @@ __device__ __forceinline__ void argmax_commit(StepState *st, int idx, int *__res
 	st->pos = st->pos + 1;
 }
 
-__global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ logits, int n, StepState *st,
+static __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ logits, int n, StepState *st,
                                                       int *__restrict__ tokens_out, int cap,
                                                       float *__restrict__ pair_out = nullptr, int index_offset = 0) {
 	float b = 0.0f;
@@ -186,7 +190,7 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float *__restrict__ 
 // then the kernel waits for every rank's pair and picks the global first max in rank order
 // (ranks own ascending slices: ties resolve to the lowest index, sampler.cpp:27-38) --
 // the exchange and the pick inside the argmax launch, identical on every rank.
-__global__ __launch_bounds__(1024) void argmax_tp_kernel(const float *__restrict__ logits, int n, StepState *st,
+static __global__ __launch_bounds__(1024) void argmax_tp_kernel(const float *__restrict__ logits, int n, StepState *st,
                                                          int *__restrict__ tokens_out, int cap, TpX t) {
 	const unsigned g = t.g();
 	float b = 0.0f;
@@ -220,7 +224,7 @@ __device__ __forceinline__ void tpx_wait_all(const TpX &t, unsigned g, int n) {
 
 // Tensor parallelism over IPC, ranks sharing one GPU: wait for the exchange in one wave
 // before the consumer launch (yalm_hip.hip tpx_consume).
-__global__ __launch_bounds__(64) void tpx_gate_kernel(TpX t, int n) {
+static __global__ __launch_bounds__(64) void tpx_gate_kernel(TpX t, int n) {
 	tpx_wait_all(t, t.g(), n);
 }
 
@@ -228,7 +232,7 @@ __global__ __launch_bounds__(64) void tpx_gate_kernel(TpX t, int n) {
 // the summed x into `out` (the collect form of many ranks, yalm_block's result, the timing
 // hook), or, with gather, the n floats of every rank's slot side by side (the sharded
 // logits). Any grid: element i belongs to global thread i mod the grid's threads.
-__global__ __launch_bounds__(256) void tpx_collect_kernel(TpX t, int n, int gather, float *__restrict__ out) {
+static __global__ __launch_bounds__(256) void tpx_collect_kernel(TpX t, int n, int gather, float *__restrict__ out) {
 	const unsigned g = t.g();
 	const unsigned long long deadline = __builtin_amdgcn_s_memrealtime() + TPX_TIMEOUT;
 	const int i0 = blockIdx.x * blockDim.x + threadIdx.x, stride = gridDim.x * blockDim.x;
@@ -248,7 +252,7 @@ __global__ __launch_bounds__(256) void tpx_collect_kernel(TpX t, int n, int gath
 
 // Timing hook (yalm_time_kernel id 6 under IPC): a producer of exchange g alone -- this
 // rank's x pushed to every rank's slot -- for the collect launch that follows.
-__global__ __launch_bounds__(1024) void tpx_push_kernel(TpX t, int n, const float *__restrict__ x) {
+static __global__ __launch_bounds__(1024) void tpx_push_kernel(TpX t, int n, const float *__restrict__ x) {
 	const unsigned g = t.g();
 	for (int i = threadIdx.x; i < n; i += blockDim.x)
 		tpx_put(t, g, i, x[i]);
@@ -257,7 +261,7 @@ __global__ __launch_bounds__(1024) void tpx_push_kernel(TpX t, int n, const floa
 // Tensor parallelism: pick the global first maximum from the tp_size gathered
 // (value, index) pairs (ranks own ascending vocab slices, so ties resolve to the
 // lowest index as in sampler.cpp:27-38) and advance the step like argmax_kernel.
-__global__ void argmax_pick_kernel(const float *__restrict__ pairs, int n_pairs, StepState *st,
+static __global__ void argmax_pick_kernel(const float *__restrict__ pairs, int n_pairs, StepState *st,
                                    int *__restrict__ tokens_out, int cap) {
 	float b = pairs[0];
 	int idx = __float_as_int(pairs[1]);
@@ -277,30 +281,4 @@ __global__ void argmax_pick_kernel(const float *__restrict__ pairs, int n_pairs,
 	st->pos = st->pos + 1;
 }
 
-// Deterministic synthetic initialiser — the same integer hash as the CPU
-// oracle (oracle/yalm_oracle.c orc_synth_*), so a random-weight model of a
-// real shape can be built in HBM and reproduced bit-exactly on the host.
-__device__ __forceinline__ uint64_t splitmix64(uint64_t x) {
-	x += 0x9E3779B97F4A7C15ull;
-	x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
-	x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
-	return x ^ (x >> 31);
-}
-
-__global__ void synth_kernel(void *dst, size_t n, int dtype, uint64_t seed, float scale, float offset) {
-	const float k = scale * (1.0f / 8388608.0f);
-	for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
-		uint64_t h = splitmix64(seed ^ ((uint64_t)i * 0xD1B54A32D192ED03ull));
-		int32_t s = (int32_t)(h >> 40) - 8388608;
-		if (dtype == 0) {
-			((float *)dst)[i] = __builtin_fmaf((float)s, k, offset);
-		} else {
-			float v = __fmul_rn((float)s, k);
-			uint32_t hb = f2h(v); // f2h keeps the f32 rounding step (no fma_mix fusion)
-			if (dtype == 1)
-				((uint16_t *)dst)[i] = (uint16_t)hb;
-			else
-				((uint8_t *)dst)[i] = (uint8_t)((hb + 0x7Fu + ((hb >> 8) & 1u)) >> 8);
-		}
-	}
-}
+#pragma clang diagnostic pop

@@ -1,0 +1,707 @@
+// seq.hip — the layer-list engine of the C ABI (include/yalm_hip.h, "layer-list models"):
+// a decoder whose layers each name their token mixer (latent attention, real-gated linear
+// recurrence, gated delta rule) and feed-forward (dense GLU, routed experts), holding one
+// sequence's latent caches and recurrent / convolution states in HBM. One step function
+// serves whole prompts, portions of prompts and single decoded tokens; the device greedy
+// loop feeds the argmax back without a host round trip, as yalm_generate_greedy does.
+#include "../../include/yalm_hip.h"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "decoder.h"
+#include "device_common.h"
+#include "misc_kernels.h"
+#include "seq_kernels.h"
+
+struct yalm_seq_s {
+	yalm_seq_config c{};
+	std::vector<yalm_seq_layer> L;
+	const void *embed = nullptr, *head = nullptr;
+	const float *final_norm = nullptr;
+	hipStream_t stream = nullptr;
+	bool own_stream = false;
+	StepState *st = nullptr;
+	int host_pos = 0;
+	int cap = 0;                 // tokens per internal portion
+	size_t bw = 0;               // floats per row of the work buffers B0..B3
+	int zw = 0;                  // floats per row of Z (the widest input projection)
+	float *X = nullptr, *Hn = nullptr, *Y = nullptr, *Z = nullptr, *B[4] = {};
+	float *inv_freq = nullptr;
+	int *tok = nullptr, *want = nullptr;
+	float *logits = nullptr;     // [LOGIT_ROWS][vocab]
+	int *idx = nullptr, *counts = nullptr, *lists = nullptr;
+	float *wt = nullptr, *sgate = nullptr;
+	float *arena = nullptr;      // every recurrent and convolution state of the sequence
+	size_t arena_floats = 0;
+	std::vector<void *> cache;   // per layer: [max_tokens][kv_rank] latent rows (own latent only)
+	std::vector<float *> S, conv;
+	float *dump = nullptr;
+	bool dump_on = false;
+	int dump_n = 0;
+	int *gen_tokens = nullptr;
+	int gen_cap = 0;
+	std::vector<void *> allocs;
+};
+typedef yalm_seq_s Seq;
+
+enum { LOGIT_ROWS = 64, SEQ_PORTION_CAP = 4096 };
+
+static int salloc(Seq *q, void **p, size_t bytes) {
+	*p = nullptr;
+	HIPCHK(hipMalloc(p, bytes ? bytes : 1));
+	q->allocs.push_back(*p);
+	HIPCHK(hipMemset(*p, 0, bytes ? bytes : 1));
+	return YALM_OK;
+}
+template <class T>
+static int sallocT(Seq *q, T **p, size_t count) {
+	return salloc(q, (void **)p, count * sizeof(T));
+}
+
+static int cdiv(int a, int b) {
+	return (a + b - 1) / b;
+}
+
+// ------------------------------------------------------------------ validation
+static int in_rows(const yalm_seq_layer &l) {
+	switch (l.mixer) {
+	case YALM_MIX_LATENT: return l.q_rank + (l.kv_from < 0 ? l.kv_rank : 0);
+	case YALM_MIX_RGLRU: return 2 * l.rec_width;
+	default: return 2 * l.kv_heads * l.dim + 2 * l.heads * l.vdim + 2 * l.heads;
+	}
+}
+
+static int validate(const yalm_seq_config &c, const std::vector<yalm_seq_layer> &L) {
+	ARGCHK(c.width > 0 && c.width % 2 == 0 && c.vocab > 0 && c.n_layers > 0 && c.max_tokens > 0,
+	       "yalm_seq_create: bad model sizes (width must be even)");
+	ARGCHK(c.weight_dtype == YALM_BF16 || c.weight_dtype == YALM_F32, "yalm_seq_create: weight_dtype must be bf16 or f32");
+	for (int i = 0; i < c.n_layers; ++i) {
+		const yalm_seq_layer &l = L[i];
+		const std::string at = "yalm_seq_create: layer " + std::to_string(i) + ": ";
+		ARGCHK(l.norm1 && l.norm1b && l.w_in && l.w_o, at + "missing tensors");
+		if (l.mixer == YALM_MIX_LATENT) {
+			ARGCHK(l.heads > 0 && l.dim > 0 && l.vdim > 0 && l.kv_rank > 0 && l.q_rank > 0, at + "bad latent attention sizes");
+			if (l.kv_rank > 256) {
+				set_err(at + "kv_rank above 256 is not implemented by the latent attention kernel");
+				return YALM_ERR_UNSUPPORTED;
+			}
+			ARGCHK(l.q_norm && l.w_uq && l.w_ukt && l.w_uv, at + "missing latent attention tensors");
+			if (l.kv_from >= 0) {
+				ARGCHK(l.kv_from < i && L[l.kv_from].mixer == YALM_MIX_LATENT && L[l.kv_from].kv_from < 0 &&
+				           L[l.kv_from].kv_rank == l.kv_rank,
+				       at + "kv_from must name an earlier latent attention layer with its own latent of the same rank");
+			} else {
+				ARGCHK(l.kv_norm, at + "missing latent norm");
+			}
+		} else if (l.mixer == YALM_MIX_RGLRU) {
+			ARGCHK(l.rec_width > 0 && l.blocks > 0 && l.rec_width % l.blocks == 0, at + "bad recurrence sizes");
+			ARGCHK(l.conv >= 1 && l.conv <= SEQ_MAX_TAPS, at + "convolution taps out of range");
+			ARGCHK(l.in_bias && l.conv_w && l.conv_b && l.gate_a && l.gate_a_b && l.gate_i && l.gate_i_b && l.lam,
+			       at + "missing recurrence tensors");
+		} else if (l.mixer == YALM_MIX_DELTA) {
+			ARGCHK(l.heads > 0 && l.kv_heads > 0 && l.heads % l.kv_heads == 0 && l.dim > 0 && l.vdim > 0,
+			       at + "bad delta rule sizes");
+			if (l.dim > 256) {
+				set_err(at + "dim above 256 is not implemented by the delta rule kernel");
+				return YALM_ERR_UNSUPPORTED;
+			}
+			ARGCHK(l.conv >= 1 && l.conv <= SEQ_MAX_TAPS, at + "convolution taps out of range");
+			ARGCHK(l.conv_w && l.a_log && l.dt_bias && l.out_norm, at + "missing delta rule tensors");
+		} else {
+			ARGCHK(false, at + "unknown mixer");
+		}
+		if (l.ff_kind == YALM_FF_DENSE) {
+			ARGCHK(l.ff > 0 && l.w_gate && l.w_up && l.w_down && l.norm2 && l.norm2b, at + "bad dense feed-forward");
+		} else if (l.ff_kind == YALM_FF_MOE) {
+			ARGCHK(l.ff > 0 && l.experts > 0 && l.top > 0 && l.top <= l.experts && l.groups > 0 &&
+			           l.groups <= SEQ_MAX_GROUPS && l.experts % l.groups == 0 && l.groups_keep > 0 &&
+			           l.groups_keep <= l.groups && l.top <= l.groups_keep * (l.experts / l.groups),
+			       at + "bad router sizes");
+			ARGCHK(l.router && l.w_gate && l.w_up && l.w_down && l.norm2 && l.norm2b, at + "missing expert tensors");
+			if (l.shared_ff > 0)
+				ARGCHK(l.ws_gate && l.ws_up && l.ws_down && l.shared_sg, at + "missing shared expert tensors");
+		} else {
+			ARGCHK(l.ff_kind == YALM_FF_NONE, at + "unknown feed-forward kind");
+		}
+	}
+	return YALM_OK;
+}
+
+// ------------------------------------------------------------------ create / destroy
+static void destroy_seq(Seq *q) {
+	for (void *p : q->allocs)
+		(void)hipFree(p);
+	if (q->own_stream && q->stream)
+		(void)hipStreamDestroy(q->stream);
+	delete q;
+}
+
+template <class CT, int NACC>
+static int att_attr(int rank) {
+	HIPCHK(hipFuncSetAttribute((const void *)seq_latent_attn_kernel<CT, NACC>, hipFuncAttributeMaxDynamicSharedMemorySize,
+	                           (int)att_lds_bytes(rank)));
+	return YALM_OK;
+}
+template <class CT>
+static int att_attr_ct(int rank) {
+	const int na = cdiv(rank, 16);
+	if (na <= 1) return att_attr<CT, 1>(rank);
+	if (na <= 2) return att_attr<CT, 2>(rank);
+	if (na <= 4) return att_attr<CT, 4>(rank);
+	if (na <= 8) return att_attr<CT, 8>(rank);
+	return att_attr<CT, 16>(rank);
+}
+
+static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, yalm_stream s, Seq **out) {
+	ARGCHK(config && w && w->layers && w->embed && w->final_norm && w->head && out, "yalm_seq_create: null argument");
+	Seq *q = new Seq;
+	q->c = *config;
+	q->L.assign(w->layers, w->layers + config->n_layers);
+	q->embed = w->embed;
+	q->head = w->head;
+	q->final_norm = w->final_norm;
+	int rc = validate(q->c, q->L);
+	if (rc != YALM_OK) {
+		delete q;
+		return rc;
+	}
+	auto fail = [&](int r) {
+		destroy_seq(q);
+		return r;
+	};
+#define STRY(expr)                                                                                                     \
+	do {                                                                                                               \
+		int r_ = (expr);                                                                                               \
+		if (r_ != YALM_OK)                                                                                             \
+			return fail(r_);                                                                                           \
+	} while (0)
+	if (s) {
+		q->stream = reinterpret_cast<hipStream_t>(s);
+	} else {
+		if (hipStreamCreateWithFlags(&q->stream, hipStreamNonBlocking) != hipSuccess) {
+			set_err("hipStreamCreateWithFlags failed");
+			return fail(YALM_ERR_HIP);
+		}
+		q->own_stream = true;
+	}
+	const yalm_seq_config &c = q->c;
+	const bool bf = c.weight_dtype == YALM_BF16;
+	q->cap = std::min(c.max_tokens, (int)SEQ_PORTION_CAP);
+	size_t bw = c.width, arena = 0;
+	int zw = 1, max_e = 1, max_top = 1;
+	for (const yalm_seq_layer &l : q->L) {
+		zw = std::max(zw, in_rows(l));
+		if (l.mixer == YALM_MIX_LATENT) {
+			bw = std::max({bw, (size_t)l.heads * l.dim, (size_t)l.heads * l.kv_rank, (size_t)l.heads * l.vdim, (size_t)l.q_rank});
+		} else if (l.mixer == YALM_MIX_RGLRU) {
+			bw = std::max(bw, (size_t)l.rec_width);
+			arena += (size_t)l.rec_width + (size_t)(l.conv - 1) * l.rec_width;
+		} else {
+			const size_t cc = 2 * (size_t)l.kv_heads * l.dim + (size_t)l.heads * l.vdim;
+			bw = std::max({bw, cc, (size_t)l.heads * l.vdim, (size_t)2 * l.heads});
+			arena += (size_t)l.heads * l.dim * l.vdim + (size_t)(l.conv - 1) * cc;
+		}
+		if (l.ff_kind == YALM_FF_DENSE)
+			bw = std::max(bw, (size_t)l.ff);
+		if (l.ff_kind == YALM_FF_MOE) {
+			bw = std::max({bw, (size_t)l.top * l.ff, (size_t)l.top * c.width, (size_t)l.shared_ff});
+			max_e = std::max(max_e, l.experts);
+			max_top = std::max(max_top, l.top);
+		}
+	}
+	q->bw = bw;
+	q->zw = zw;
+	const size_t cap = q->cap;
+	STRY(sallocT(q, &q->st, 1));
+	STRY(sallocT(q, &q->X, cap * c.width));
+	STRY(sallocT(q, &q->Hn, cap * c.width));
+	STRY(sallocT(q, &q->Y, cap * c.width));
+	STRY(sallocT(q, &q->Z, cap * zw));
+	for (int i = 0; i < 4; ++i)
+		STRY(sallocT(q, &q->B[i], cap * bw));
+	STRY(sallocT(q, &q->tok, cap));
+	STRY(sallocT(q, &q->want, cap));
+	STRY(sallocT(q, &q->logits, (size_t)LOGIT_ROWS * c.vocab));
+	STRY(sallocT(q, &q->idx, cap * max_top));
+	STRY(sallocT(q, &q->wt, cap * max_top));
+	STRY(sallocT(q, &q->sgate, cap));
+	STRY(sallocT(q, &q->counts, max_e));
+	STRY(sallocT(q, &q->lists, (size_t)max_e * cap));
+	q->gen_cap = 1 << 16;
+	STRY(sallocT(q, &q->gen_tokens, q->gen_cap));
+	// position frequencies 10000^(-2 i / width), evaluated in double
+	{
+		std::vector<float> f(c.width / 2);
+		for (int i = 0; i < c.width / 2; ++i)
+			f[i] = (float)std::pow(10000.0, -2.0 * i / (double)c.width);
+		STRY(sallocT(q, &q->inv_freq, f.size()));
+		if (hipMemcpy(q->inv_freq, f.data(), f.size() * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) {
+			set_err("hipMemcpy of the position frequencies failed");
+			return fail(YALM_ERR_HIP);
+		}
+	}
+	q->arena_floats = arena;
+	STRY(sallocT(q, &q->arena, arena));
+	q->cache.assign(c.n_layers, nullptr);
+	q->S.assign(c.n_layers, nullptr);
+	q->conv.assign(c.n_layers, nullptr);
+	size_t off = 0;
+	for (int i = 0; i < c.n_layers; ++i) {
+		const yalm_seq_layer &l = q->L[i];
+		if (l.mixer == YALM_MIX_LATENT) {
+			if (l.kv_from < 0)
+				STRY(salloc(q, &q->cache[i], (size_t)c.max_tokens * l.kv_rank * (bf ? 2 : 4)));
+			STRY(bf ? att_attr_ct<uint16_t>(l.kv_rank) : att_attr_ct<float>(l.kv_rank));
+		} else if (l.mixer == YALM_MIX_RGLRU) {
+			q->S[i] = q->arena + off;
+			off += l.rec_width;
+			q->conv[i] = q->arena + off;
+			off += (size_t)(l.conv - 1) * l.rec_width;
+		} else {
+			const size_t cc = 2 * (size_t)l.kv_heads * l.dim + (size_t)l.heads * l.vdim;
+			q->S[i] = q->arena + off;
+			off += (size_t)l.heads * l.dim * l.vdim;
+			q->conv[i] = q->arena + off;
+			off += (size_t)(l.conv - 1) * cc;
+		}
+	}
+	for (int i = 0; i < c.n_layers; ++i)
+		if (q->L[i].mixer == YALM_MIX_LATENT && q->L[i].kv_from >= 0)
+			q->cache[i] = q->cache[q->L[i].kv_from];
+#undef STRY
+	*out = q;
+	return YALM_OK;
+}
+
+extern "C" int yalm_seq_create(const yalm_seq_config *config, const yalm_seq_weights *weights, yalm_stream s,
+                               yalm_seq *out) {
+	Seq *q = nullptr;
+	TRY(create_seq(config, weights, s, &q));
+	*out = q;
+	return YALM_OK;
+}
+
+extern "C" int yalm_seq_destroy(yalm_seq q) {
+	if (!q)
+		return YALM_OK;
+	(void)hipStreamSynchronize(q->stream);
+	destroy_seq(q);
+	return YALM_OK;
+}
+
+extern "C" int yalm_seq_reset(yalm_seq q) {
+	ARGCHK(q, "yalm_seq_reset: null decoder");
+	if (q->arena_floats) {
+		seq_fill_float_kernel<<<256, 256, 0, q->stream>>>(q->arena, q->arena_floats, 0.0f);
+		HIPCHK(hipGetLastError());
+	}
+	q->host_pos = 0;
+	return YALM_OK;
+}
+
+extern "C" int yalm_seq_pos(yalm_seq q, int *pos) {
+	ARGCHK(q && pos, "yalm_seq_pos: null argument");
+	*pos = q->host_pos;
+	return YALM_OK;
+}
+
+// ------------------------------------------------------------------ launches
+template <class WT>
+static int gemm_t(Seq *q, const GemmArgs &a, int batches, int max_m) {
+	const bool glu = a.W2 != nullptr;
+	if (max_m <= GEMV_MAX_M) {
+		const dim3 g(cdiv(a.N, SEQ_THREADS / 64), 1, batches);
+		if (glu)
+			seq_gemv_kernel<WT, true><<<g, SEQ_THREADS, 0, q->stream>>>(a);
+		else
+			seq_gemv_kernel<WT, false><<<g, SEQ_THREADS, 0, q->stream>>>(a);
+	} else {
+		const dim3 g(cdiv(a.N, GT_BN), cdiv(max_m, GT_BM), batches);
+		if (glu)
+			seq_gemm_kernel<WT, true><<<g, SEQ_THREADS, 0, q->stream>>>(a);
+		else
+			seq_gemm_kernel<WT, false><<<g, SEQ_THREADS, 0, q->stream>>>(a);
+	}
+	HIPCHK(hipGetLastError());
+	return YALM_OK;
+}
+// f32w: the matrices are f32 whatever the model's weight type (the recurrence's gates)
+static int gemm(Seq *q, const GemmArgs &a, int batches = 1, int max_m = -1, bool f32w = false) {
+	if (max_m < 0)
+		max_m = a.M;
+	if (f32w || q->c.weight_dtype == YALM_F32)
+		return gemm_t<WF32>(q, a, batches, max_m);
+	return gemm_t<WBF16>(q, a, batches, max_m);
+}
+static GemmArgs plain(const float *A, int lda, const void *W, int ldw, float *C, int ldc, int M, int N, int K) {
+	GemmArgs a;
+	a.A = A;
+	a.lda = lda;
+	a.W = W;
+	a.ldw = ldw;
+	a.C = C;
+	a.ldc = ldc;
+	a.M = M;
+	a.N = N;
+	a.K = K;
+	return a;
+}
+
+template <class CT>
+static int attn_t(Seq *q, const float *Qa, const void *cache, int rank, int H, int n, float scale, float *ctx) {
+	const int NR = n * H;
+	const dim3 g(cdiv(NR, ATT_BR));
+	const size_t lds = att_lds_bytes(rank);
+	const int na = cdiv(rank, 16);
+#define ATT_LAUNCH(NA)                                                                                                 \
+	seq_latent_attn_kernel<CT, NA><<<g, SEQ_THREADS, lds, q->stream>>>(Qa, (const CT *)cache, rank, H, NR, scale, q->st, ctx)
+	if (na <= 1) ATT_LAUNCH(1);
+	else if (na <= 2) ATT_LAUNCH(2);
+	else if (na <= 4) ATT_LAUNCH(4);
+	else if (na <= 8) ATT_LAUNCH(8);
+	else ATT_LAUNCH(16);
+#undef ATT_LAUNCH
+	HIPCHK(hipGetLastError());
+	return YALM_OK;
+}
+
+static int mixer_latent(Seq *q, int li, int n) {
+	const yalm_seq_layer &l = q->L[li];
+	const yalm_seq_config &c = q->c;
+	const bool bf = c.weight_dtype == YALM_BF16;
+	const int zin = in_rows(l), H = l.heads, D = l.dim, V = l.vdim, rk = l.kv_rank;
+	float *cq = q->B[0], *qh = q->B[1], *qa = q->B[2], *ctx = q->B[3];
+	TRY(gemm(q, plain(q->Hn, c.width, l.w_in, c.width, q->Z, zin, n, zin, c.width)));
+	seq_norm_kernel<float><<<n, SEQ_THREADS, 0, q->stream>>>(q->Z, zin, l.q_norm, c.norm_eps, l.q_rank, cq, l.q_rank,
+	                                                         nullptr, q->st, 0);
+	if (l.kv_from < 0) {
+		if (bf)
+			seq_norm_kernel<uint16_t><<<n, SEQ_THREADS, 0, q->stream>>>(q->Z + l.q_rank, zin, l.kv_norm, c.norm_eps, rk,
+			                                                            (uint16_t *)q->cache[li], rk, nullptr, q->st, 1);
+		else
+			seq_norm_kernel<float><<<n, SEQ_THREADS, 0, q->stream>>>(q->Z + l.q_rank, zin, l.kv_norm, c.norm_eps, rk,
+			                                                         (float *)q->cache[li], rk, nullptr, q->st, 1);
+	}
+	HIPCHK(hipGetLastError());
+	TRY(gemm(q, plain(cq, l.q_rank, l.w_uq, l.q_rank, qh, H * D, n, H * D, l.q_rank)));
+	{ // q~[h] = W_uk[h]^T q[h]: per head [n][dim] x [rank][dim]^T
+		GemmArgs a = plain(qh, H * D, l.w_ukt, D, qa, H * rk, n, rk, D);
+		a.a_bs = D;
+		a.w_bs = (long)rk * D;
+		a.c_bs = rk;
+		TRY(gemm(q, a, H));
+	}
+	TRY(bf ? attn_t<uint16_t>(q, qa, q->cache[li], rk, H, n, l.attn_scale, ctx)
+	       : attn_t<float>(q, qa, q->cache[li], rk, H, n, l.attn_scale, ctx));
+	{ // o[h] = W_uv[h] ctx[h]
+		GemmArgs a = plain(ctx, H * rk, l.w_uv, rk, qh, H * V, n, V, rk);
+		a.a_bs = rk;
+		a.w_bs = (long)V * rk;
+		a.c_bs = V;
+		TRY(gemm(q, a, H));
+	}
+	return gemm(q, plain(qh, H * V, l.w_o, H * V, q->Y, c.width, n, c.width, H * V));
+}
+
+static int conv_launch(Seq *q, const float *Z, int ldz, int col0, int C, int taps, const float *w, const float *bias,
+                       int silu, float *state, float *out, int n) {
+	seq_conv_kernel<<<dim3(cdiv(C, SEQ_THREADS), n), SEQ_THREADS, 0, q->stream>>>(Z, ldz, col0, C, taps, w, bias, silu,
+	                                                                              state, out, C, n);
+	if (taps > 1)
+		seq_conv_state_kernel<<<cdiv(C, SEQ_THREADS), SEQ_THREADS, 0, q->stream>>>(Z, ldz, col0, C, taps, state, n);
+	HIPCHK(hipGetLastError());
+	return YALM_OK;
+}
+
+static int mixer_rglru(Seq *q, int li, int n) {
+	const yalm_seq_layer &l = q->L[li];
+	const yalm_seq_config &c = q->c;
+	const int W = l.rec_width, bs = W / l.blocks;
+	float *u = q->B[0], *r = q->B[1], *ig = q->B[2], *so = q->B[3];
+	{
+		GemmArgs a = plain(q->Hn, c.width, l.w_in, c.width, q->Z, 2 * W, n, 2 * W, c.width);
+		a.bias = l.in_bias;
+		TRY(gemm(q, a));
+	}
+	TRY(conv_launch(q, q->Z, 2 * W, W, W, l.conv, l.conv_w, l.conv_b, 0, q->conv[li], u, n));
+	for (int g = 0; g < 2; ++g) { // block-diagonal gates in f32
+		GemmArgs a = plain(u, W, g ? l.gate_i : l.gate_a, bs, g ? ig : r, W, n, bs, bs);
+		a.a_bs = bs;
+		a.w_bs = (long)bs * bs;
+		a.c_bs = bs;
+		a.bias = g ? l.gate_i_b : l.gate_a_b;
+		a.bias_bs = bs;
+		a.epi = EPI_SIGMOID;
+		TRY(gemm(q, a, l.blocks, -1, true));
+	}
+	seq_rglru_scan_kernel<<<cdiv(W, SEQ_THREADS), SEQ_THREADS, 0, q->stream>>>(r, ig, u, W, q->Z, 2 * W, l.lam, q->S[li],
+	                                                                           so, n);
+	HIPCHK(hipGetLastError());
+	return gemm(q, plain(so, W, l.w_o, W, q->Y, c.width, n, c.width, W));
+}
+
+static int mixer_delta(Seq *q, int li, int n) {
+	const yalm_seq_layer &l = q->L[li];
+	const yalm_seq_config &c = q->c;
+	const int H = l.heads, KH = l.kv_heads, D = l.dim, V = l.vdim;
+	const int CQ = KH * D, CV = H * V, cc = 2 * CQ + CV, zin = in_rows(l);
+	const int gcol = cc, bcol = cc + CV, acol = bcol + H;
+	float *qkv = q->B[0], *bg = q->B[1], *o = q->B[2], *on = q->B[3];
+	TRY(gemm(q, plain(q->Hn, c.width, l.w_in, c.width, q->Z, zin, n, zin, c.width)));
+	TRY(conv_launch(q, q->Z, zin, 0, cc, l.conv, l.conv_w, nullptr, 1, q->conv[li], qkv, n));
+	seq_delta_prep_kernel<<<n, SEQ_THREADS, 0, q->stream>>>(qkv, cc, KH, D, q->Z, zin, bcol, acol, H, l.a_log, l.dt_bias,
+	                                                        bg);
+	const dim3 g(cdiv(V, SEQ_THREADS / 8), H);
+	const int R = cdiv(D, 8);
+#define DELTA_LAUNCH(RR) seq_delta_kernel<RR><<<g, SEQ_THREADS, 0, q->stream>>>(qkv, cc, KH, D, H, V, bg, q->S[li], o, n)
+	if (R <= 4) DELTA_LAUNCH(4);
+	else if (R <= 8) DELTA_LAUNCH(8);
+	else if (R <= 16) DELTA_LAUNCH(16);
+	else DELTA_LAUNCH(32);
+#undef DELTA_LAUNCH
+	seq_delta_out_kernel<<<n, SEQ_THREADS, 0, q->stream>>>(o, H, V, l.out_norm, c.norm_eps, q->Z, zin, gcol, on);
+	HIPCHK(hipGetLastError());
+	return gemm(q, plain(on, CV, l.w_o, CV, q->Y, c.width, n, c.width, CV));
+}
+
+static int ff_dense(Seq *q, int li, int n) {
+	const yalm_seq_layer &l = q->L[li];
+	const yalm_seq_config &c = q->c;
+	GemmArgs a = plain(q->Hn, c.width, l.w_gate, c.width, q->B[0], l.ff, n, l.ff, c.width);
+	a.W2 = l.w_up;
+	a.epi = EPI_GLU_GELU;
+	TRY(gemm(q, a));
+	return gemm(q, plain(q->B[0], l.ff, l.w_down, l.ff, q->Y, c.width, n, c.width, l.ff));
+}
+
+static int ff_moe(Seq *q, int li, int n) {
+	const yalm_seq_layer &l = q->L[li];
+	const yalm_seq_config &c = q->c;
+	const int E = l.experts, top = l.top, ff = l.ff, slots = n * top;
+	float *hx = q->B[0], *yx = q->B[1], *hs = q->B[2], *ys = q->B[3];
+	seq_router_kernel<<<n, SEQ_THREADS, E * sizeof(float), q->stream>>>(q->Hn, c.width, l.router, E, top, l.groups,
+	                                                                    l.groups_keep, l.router_scale,
+	                                                                    l.shared_ff > 0 ? l.shared_sg : nullptr, q->idx,
+	                                                                    q->wt, q->sgate);
+	HIPCHK(hipGetLastError());
+	if (n <= GEMV_MAX_M) { // one batch per (token, choice): its expert's matrices picked on the device
+		GemmArgs a = plain(q->Hn, c.width, l.w_gate, c.width, hx, ff, 1, ff, c.width);
+		a.W2 = l.w_up;
+		a.a_bs = c.width;
+		a.a_zdiv = top;
+		a.w_sel = q->idx;
+		a.w_bs = (long)ff * c.width;
+		a.c_bs = ff;
+		a.epi = EPI_GLU_CLAMP;
+		a.limit = l.limit;
+		TRY(gemm(q, a, slots));
+		GemmArgs b = plain(hx, ff, l.w_down, ff, yx, c.width, 1, c.width, ff);
+		b.a_bs = ff;
+		b.w_sel = q->idx;
+		b.w_bs = (long)c.width * ff;
+		b.c_bs = c.width;
+		TRY(gemm(q, b, slots));
+	} else { // tokens grouped by expert: one batch per expert over its row list
+		seq_fill_int_kernel<<<cdiv(E, 256), 256, 0, q->stream>>>(q->counts, E, 0);
+		seq_moe_lists_kernel<<<cdiv(slots, SEQ_THREADS), SEQ_THREADS, 0, q->stream>>>(q->idx, slots, q->counts, q->lists,
+		                                                                              q->cap);
+		HIPCHK(hipGetLastError());
+		GemmArgs a = plain(q->Hn, c.width, l.w_gate, c.width, hx, ff, n, ff, c.width);
+		a.W2 = l.w_up;
+		a.w_bs = (long)ff * c.width;
+		a.rows = q->lists;
+		a.rows_bs = q->cap;
+		a.counts = q->counts;
+		a.a_div = top;
+		a.epi = EPI_GLU_CLAMP;
+		a.limit = l.limit;
+		TRY(gemm(q, a, E, n));
+		GemmArgs b = plain(hx, ff, l.w_down, ff, yx, c.width, n, c.width, ff);
+		b.w_bs = (long)c.width * ff;
+		b.rows = q->lists;
+		b.rows_bs = q->cap;
+		b.counts = q->counts;
+		TRY(gemm(q, b, E, n));
+	}
+	if (l.shared_ff > 0) {
+		GemmArgs a = plain(q->Hn, c.width, l.ws_gate, c.width, hs, l.shared_ff, n, l.shared_ff, c.width);
+		a.W2 = l.ws_up;
+		a.epi = EPI_GLU_CLAMP;
+		a.limit = l.shared_limit;
+		TRY(gemm(q, a));
+		TRY(gemm(q, plain(hs, l.shared_ff, l.ws_down, l.shared_ff, ys, c.width, n, c.width, l.shared_ff)));
+	}
+	seq_moe_combine_kernel<<<dim3(cdiv(c.width, SEQ_THREADS), n), SEQ_THREADS, 0, q->stream>>>(
+	    yx, q->wt, top, l.shared_ff > 0 ? ys : nullptr, q->sgate, c.width, q->Y);
+	HIPCHK(hipGetLastError());
+	return YALM_OK;
+}
+
+static int add_norm(Seq *q, const float *wb, const float *w_next, int n) {
+	seq_add_norm_kernel<<<n, SEQ_THREADS, q->c.width * sizeof(float), q->stream>>>(q->X, q->Y, wb, q->c.norm_eps,
+	                                                                               q->c.width, w_next, q->Hn);
+	HIPCHK(hipGetLastError());
+	return YALM_OK;
+}
+
+// One portion of n <= cap tokens through every layer, from the states and caches earlier
+// portions left; tokens_dev == nullptr: the greedy loop's device-resident token. The
+// position is st->pos on the device (set by the caller).
+static int enqueue_portion(Seq *q, const int *tokens_dev, int n) {
+	const yalm_seq_config &c = q->c;
+	if (c.weight_dtype == YALM_F32)
+		seq_embed_kernel<WF32><<<n, SEQ_THREADS, 0, q->stream>>>(q->st, tokens_dev, q->embed, q->inv_freq, c.width,
+		                                                         c.vocab, c.embed_scale, q->X);
+	else
+		seq_embed_kernel<WBF16><<<n, SEQ_THREADS, 0, q->stream>>>(q->st, tokens_dev, q->embed, q->inv_freq, c.width,
+		                                                          c.vocab, c.embed_scale, q->X);
+	seq_norm_kernel<float><<<n, SEQ_THREADS, 0, q->stream>>>(q->X, c.width, q->L[0].norm1, c.norm_eps, c.width, q->Hn,
+	                                                         c.width, nullptr, q->st, 0);
+	HIPCHK(hipGetLastError());
+	for (int li = 0; li < c.n_layers; ++li) {
+		const yalm_seq_layer &l = q->L[li];
+		const float *next = li + 1 < c.n_layers ? q->L[li + 1].norm1 : nullptr;
+		if (l.mixer == YALM_MIX_LATENT)
+			TRY(mixer_latent(q, li, n));
+		else if (l.mixer == YALM_MIX_RGLRU)
+			TRY(mixer_rglru(q, li, n));
+		else
+			TRY(mixer_delta(q, li, n));
+		if (l.ff_kind == YALM_FF_NONE) {
+			TRY(add_norm(q, l.norm1b, next, n));
+		} else {
+			TRY(add_norm(q, l.norm1b, l.norm2, n));
+			TRY(l.ff_kind == YALM_FF_DENSE ? ff_dense(q, li, n) : ff_moe(q, li, n));
+			TRY(add_norm(q, l.norm2b, next, n));
+		}
+		if (q->dump_on && q->dump)
+			HIPCHK(hipMemcpyAsync(q->dump + (size_t)li * n * c.width, q->X, (size_t)n * c.width * sizeof(float),
+			                      hipMemcpyDeviceToDevice, q->stream));
+	}
+	return YALM_OK;
+}
+
+// Final norm of the asked rows and their logits into q->logits ([n_rows][vocab], n_rows <= LOGIT_ROWS).
+static int enqueue_logits(Seq *q, const int *rows_dev, int n_rows) {
+	const yalm_seq_config &c = q->c;
+	seq_norm_kernel<float><<<n_rows, SEQ_THREADS, 0, q->stream>>>(q->X, c.width, q->final_norm, c.norm_eps, c.width,
+	                                                              q->Hn, c.width, rows_dev, q->st, 0);
+	HIPCHK(hipGetLastError());
+	return gemm(q, plain(q->Hn, c.width, q->head, c.width, q->logits, c.vocab, n_rows, c.vocab, c.width));
+}
+
+extern "C" int yalm_seq_step(yalm_seq q, const int *tokens, int n, const int *want, int n_want, float *logits_host) {
+	ARGCHK(q && tokens && n > 0, "yalm_seq_step: null decoder or no tokens");
+	ARGCHK(n_want == 0 || (want && logits_host), "yalm_seq_step: logits asked for without a buffer");
+	ARGCHK(q->host_pos + n <= q->c.max_tokens, "yalm_seq_step: the sequence would pass max_tokens");
+	for (int i = 0; i < n_want; ++i)
+		ARGCHK(want[i] >= 0 && want[i] < n && (i == 0 || want[i] > want[i - 1]), "yalm_seq_step: want must ascend within the tokens");
+	const yalm_seq_config &c = q->c;
+	int wi = 0;
+	q->dump_n = 0;
+	for (int t0 = 0; t0 < n; t0 += q->cap) {
+		const int m = std::min(q->cap, n - t0);
+		HIPCHK(hipMemcpyAsync(q->tok, tokens + t0, (size_t)m * sizeof(int), hipMemcpyHostToDevice, q->stream));
+		set_step_kernel<<<1, 1, 0, q->stream>>>(q->st, 0, q->host_pos, 0);
+		HIPCHK(hipGetLastError());
+		if (q->dump_on) {
+			if (!q->dump)
+				TRY(sallocT(q, &q->dump, (size_t)c.n_layers * q->cap * c.width));
+			q->dump_n = m;
+		}
+		TRY(enqueue_portion(q, q->tok, m));
+		q->host_pos += m;
+		int w1 = wi;
+		while (w1 < n_want && want[w1] < t0 + m)
+			++w1;
+		while (wi < w1) { // this portion's asked rows, LOGIT_ROWS at a time
+			const int k = std::min(w1 - wi, (int)LOGIT_ROWS);
+			std::vector<int> rel(k);
+			for (int i = 0; i < k; ++i)
+				rel[i] = want[wi + i] - t0;
+			HIPCHK(hipMemcpyAsync(q->want, rel.data(), (size_t)k * sizeof(int), hipMemcpyHostToDevice, q->stream));
+			HIPCHK(hipStreamSynchronize(q->stream)); // rel leaves scope
+			TRY(enqueue_logits(q, q->want, k));
+			HIPCHK(hipMemcpyAsync(logits_host + (size_t)wi * c.vocab, q->logits, (size_t)k * c.vocab * sizeof(float),
+			                      hipMemcpyDeviceToHost, q->stream));
+			HIPCHK(hipStreamSynchronize(q->stream));
+			wi += k;
+		}
+	}
+	if (n_want)
+		HIPCHK(hipStreamSynchronize(q->stream));
+	return YALM_OK;
+}
+
+extern "C" int yalm_seq_generate_greedy(yalm_seq q, int token, int n_steps, int *out_tokens) {
+	ARGCHK(q && out_tokens && n_steps > 0 && n_steps <= q->gen_cap, "yalm_seq_generate_greedy: bad argument");
+	ARGCHK(q->host_pos + n_steps <= q->c.max_tokens, "yalm_seq_generate_greedy: the sequence would pass max_tokens");
+	ARGCHK(token >= 0 && token < q->c.vocab, "yalm_seq_generate_greedy: token out of range");
+	set_step_kernel<<<1, 1, 0, q->stream>>>(q->st, token, q->host_pos, 1);
+	seq_fill_int_kernel<<<1, 1, 0, q->stream>>>(q->want, 1, 0);
+	HIPCHK(hipGetLastError());
+	for (int i = 0; i < n_steps; ++i) {
+		TRY(enqueue_portion(q, nullptr, 1));
+		TRY(enqueue_logits(q, q->want, 1));
+		argmax_kernel<<<1, 1024, 0, q->stream>>>(q->logits, q->c.vocab, q->st, q->gen_tokens, q->gen_cap);
+		HIPCHK(hipGetLastError());
+	}
+	HIPCHK(hipMemcpyAsync(out_tokens, q->gen_tokens, (size_t)n_steps * sizeof(int), hipMemcpyDeviceToHost, q->stream));
+	HIPCHK(hipStreamSynchronize(q->stream));
+	q->host_pos += n_steps;
+	return YALM_OK;
+}
+
+extern "C" int yalm_seq_layer_dump(yalm_seq q, int on) {
+	ARGCHK(q, "yalm_seq_layer_dump: null decoder");
+	q->dump_on = on != 0;
+	return YALM_OK;
+}
+
+extern "C" int yalm_seq_get_layers(yalm_seq q, float *host, size_t count) {
+	ARGCHK(q && host, "yalm_seq_get_layers: null argument");
+	ARGCHK(q->dump && count == (size_t)q->c.n_layers * q->dump_n * q->c.width,
+	       "yalm_seq_get_layers: count must be n_layers * tokens of the last portion * width");
+	HIPCHK(hipStreamSynchronize(q->stream));
+	HIPCHK(hipMemcpy(host, q->dump, count * sizeof(float), hipMemcpyDeviceToHost));
+	return YALM_OK;
+}
+
+extern "C" int yalm_seq_time_step(yalm_seq q, int n, int pos0, int iters, float *avg_ms) {
+	ARGCHK(q && avg_ms && n > 0 && n <= q->cap && iters > 0 && pos0 >= 0 && pos0 + n <= q->c.max_tokens,
+	       "yalm_seq_time_step: bad argument");
+	std::vector<int> tk(n);
+	for (int i = 0; i < n; ++i)
+		tk[i] = (int)(((unsigned)i * 2654435761u) % (unsigned)q->c.vocab);
+	HIPCHK(hipMemcpy(q->tok, tk.data(), (size_t)n * sizeof(int), hipMemcpyHostToDevice));
+	seq_fill_int_kernel<<<1, 1, 0, q->stream>>>(q->want, 1, n - 1);
+	hipEvent_t e0, e1;
+	HIPCHK(hipEventCreate(&e0));
+	HIPCHK(hipEventCreate(&e1));
+	int rc = YALM_OK;
+	for (int it = -1; it < iters && rc == YALM_OK; ++it) { // one untimed run first
+		if (it == 0)
+			(void)hipEventRecord(e0, q->stream);
+		set_step_kernel<<<1, 1, 0, q->stream>>>(q->st, 0, pos0, 0);
+		rc = enqueue_portion(q, q->tok, n);
+		if (rc == YALM_OK)
+			rc = enqueue_logits(q, q->want, 1);
+	}
+	(void)hipEventRecord(e1, q->stream);
+	hipError_t e = hipEventSynchronize(e1);
+	float ms = 0.0f;
+	if (e == hipSuccess)
+		e = hipEventElapsedTime(&ms, e0, e1);
+	(void)hipEventDestroy(e0);
+	(void)hipEventDestroy(e1);
+	TRY(rc);
+	HIPCHK(e);
+	*avg_ms = ms / iters;
+	return YALM_OK;
+}

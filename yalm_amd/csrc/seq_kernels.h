@@ -1,0 +1,896 @@
+// seq_kernels.h — device kernels of the layer-list engine (seq.hip).
+//
+// Everything outside the matrix products is f32: the residual stream, norms, attention
+// scores and weights, routers, gates and states of the recurrences. Matrix products take
+// their weights as WT (WBF16 or WF32, device_common.h) and accumulate in f32; portions of
+// more than GEMV_MAX_M tokens run on the MFMA units with the activations rounded to bf16
+// (WBF16) or as f32 FMA tiles (WF32), single tokens and short portions as weight-streaming
+// GEMVs that keep the activations in f32. All sizes are runtime arguments.
+#pragma once
+
+#include <float.h>
+#include <math.h>
+
+#include "device_common.h"
+
+#define SEQ_THREADS 256
+
+// ------------------------------------------------------------------ scalar helpers
+__device__ __forceinline__ float sq_sigmoid(float z) {
+	return 1.0f / (1.0f + expf(-z));
+}
+__device__ __forceinline__ float sq_silu(float z) {
+	return z / (1.0f + expf(-z));
+}
+__device__ __forceinline__ float sq_softplus(float z) {
+	return z > 20.0f ? z : log1pf(expf(z));
+}
+__device__ __forceinline__ float sq_gelu_tanh(float z) {
+	return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+__device__ __forceinline__ uint16_t f2bf(float x) { // round to nearest even
+	const uint32_t u = __builtin_bit_cast(uint32_t, x);
+	return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+__device__ __forceinline__ float bf2f(uint16_t b) {
+	return __builtin_bit_cast(float, (uint32_t)b << 16);
+}
+template <class WT>
+__device__ __forceinline__ float wload(const void *W, size_t i) {
+	if constexpr (WT::BYTES == 4)
+		return ((const float *)W)[i];
+	else
+		return bf2f(((const uint16_t *)W)[i]);
+}
+
+// Sum over the workgroup (SEQ_THREADS threads); red: SEQ_THREADS / 64 floats of LDS.
+__device__ __forceinline__ float block_sum(float v, float *red) {
+	v = wave_sum(v);
+	__syncthreads();
+	if ((threadIdx.x & 63) == 0)
+		red[threadIdx.x >> 6] = v;
+	__syncthreads();
+	float t = 0.0f;
+#pragma unroll
+	for (int i = 0; i < SEQ_THREADS / 64; ++i)
+		t += red[i];
+	return t;
+}
+
+// ------------------------------------------------------------------ embedding
+// X[t] = embed[token] * scale + the interleaved (sin, cos) position vector of position
+// st->pos + t; tokens == nullptr: the single device-resident token of the greedy loop.
+template <class WT>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_embed_kernel(const StepState *__restrict__ st,
+                                                                const int *__restrict__ tokens,
+                                                                const void *__restrict__ emb,
+                                                                const float *__restrict__ inv_freq, int width,
+                                                                int vocab, float scale, float *__restrict__ X) {
+	const int t = blockIdx.x;
+	int tok = tokens ? tokens[t] : st->token;
+	tok = min(max(tok, 0), vocab - 1);
+	const float p = (float)(st->pos + t);
+	for (int i = threadIdx.x; i < width; i += SEQ_THREADS) {
+		const float ang = p * inv_freq[i >> 1];
+		const float pe = (i & 1) ? cosf(ang) : sinf(ang);
+		X[(size_t)t * width + i] = wload<WT>(emb, (size_t)tok * width + i) * scale + pe;
+	}
+}
+
+// ------------------------------------------------------------------ norms
+// out[row(t)] = in[t] / sqrt(mean(in[t]^2) + eps) * w, one workgroup per row. rows != null:
+// the input row is rows[t] (gather). pos_rows: the output row is st->pos + t (a cache write).
+template <class OT>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_norm_kernel(const float *__restrict__ in, int ld_in,
+                                                               const float *__restrict__ w, float eps, int n,
+                                                               OT *__restrict__ out, int ld_out,
+                                                               const int *__restrict__ rows,
+                                                               const StepState *__restrict__ st, int pos_rows) {
+	__shared__ float red[SEQ_THREADS / 64];
+	const int t = blockIdx.x;
+	const float *x = in + (size_t)(rows ? rows[t] : t) * ld_in;
+	float ss = 0.0f;
+	for (int i = threadIdx.x; i < n; i += SEQ_THREADS)
+		ss = fmaf(x[i], x[i], ss);
+	ss = block_sum(ss, red);
+	const float r = 1.0f / sqrtf(ss / (float)n + eps);
+	OT *o = out + (size_t)(pos_rows ? st->pos + t : t) * ld_out;
+	for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
+		const float v = x[i] * r * w[i];
+		if constexpr (sizeof(OT) == 2)
+			o[i] = f2bf(v);
+		else
+			o[i] = v;
+	}
+}
+
+// The seam between two sublayers in one launch: X[t] += norm(Y[t]) * wb (the closing norm
+// of the sublayer that produced Y and the residual sum), then, if w_next, Hn[t] =
+// norm(X[t]) * w_next (the opening norm of the next sublayer). Dynamic LDS: n floats.
+__global__ __launch_bounds__(SEQ_THREADS) void seq_add_norm_kernel(float *__restrict__ X, const float *__restrict__ Y,
+                                                                   const float *__restrict__ wb, float eps, int n,
+                                                                   const float *__restrict__ w_next,
+                                                                   float *__restrict__ Hn) {
+	extern __shared__ float row[];
+	__shared__ float red[SEQ_THREADS / 64];
+	const int t = blockIdx.x;
+	const float *y = Y + (size_t)t * n;
+	float *x = X + (size_t)t * n;
+	float ss = 0.0f;
+	for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
+		const float v = y[i];
+		row[i] = v;
+		ss = fmaf(v, v, ss);
+	}
+	ss = block_sum(ss, red);
+	const float r = 1.0f / sqrtf(ss / (float)n + eps);
+	float s2 = 0.0f;
+	for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
+		const float v = x[i] + row[i] * r * wb[i];
+		x[i] = v;
+		row[i] = v;
+		s2 = fmaf(v, v, s2);
+	}
+	if (!w_next)
+		return;
+	s2 = block_sum(s2, red);
+	const float r2 = 1.0f / sqrtf(s2 / (float)n + eps);
+	for (int i = threadIdx.x; i < n; i += SEQ_THREADS)
+		Hn[(size_t)t * n + i] = row[i] * r2 * w_next[i];
+}
+
+// ------------------------------------------------------------------ matrix products
+enum { EPI_NONE = 0, EPI_GLU_GELU = 1, EPI_GLU_CLAMP = 2, EPI_SIGMOID = 3 };
+
+// C[c_row(m)][n] = epi(sum_k A[a_row(m)][k] W[n][k]) for every batch z = blockIdx.z.
+struct GemmArgs {
+	const float *A = nullptr;
+	int lda = 0;
+	long a_bs = 0;  // A offset per batch (elements)
+	int a_zdiv = 0; // > 0: the A batch offset is (z / a_zdiv) * a_bs
+	const void *W = nullptr, *W2 = nullptr; // W2: the second matrix of a GLU pair (same geometry)
+	int ldw = 0;
+	long w_bs = 0;
+	const int *w_sel = nullptr; // != null: batch z reads matrix w_sel[z]
+	float *C = nullptr;
+	int ldc = 0;
+	long c_bs = 0;
+	const float *bias = nullptr;
+	long bias_bs = 0;
+	int M = 0, N = 0, K = 0;
+	const int *rows = nullptr; // != null: row list of batch z at rows + z * rows_bs, its length counts[z]
+	long rows_bs = 0;
+	const int *counts = nullptr;
+	int a_div = 1;   // A row = list entry / a_div
+	int c_dense = 0; // 1: C row = m, 0: C row = list entry
+	int epi = EPI_NONE;
+	float limit = 0.0f;
+};
+
+__device__ __forceinline__ float epi_apply(const GemmArgs &a, float v, float v2, float b) {
+	switch (a.epi) {
+	case EPI_GLU_GELU: return sq_gelu_tanh(v) * v2;
+	case EPI_GLU_CLAMP: {
+		const float g = fminf(v, a.limit);
+		const float u = fminf(fmaxf(v2, -a.limit), a.limit);
+		return g * sq_sigmoid(1.702f * g) * (u + 1.0f);
+	}
+	case EPI_SIGMOID: return sq_sigmoid(v + b);
+	default: return v + b;
+	}
+}
+
+struct GemmBatch {
+	const float *A;
+	const char *W, *W2;
+	float *C;
+	const float *bias;
+	const int *rows;
+	int M;
+};
+template <class WT>
+__device__ __forceinline__ GemmBatch gemm_batch(const GemmArgs &a, int z) {
+	GemmBatch b;
+	const long za = a.a_zdiv > 0 ? z / a.a_zdiv : z;
+	b.A = a.A + za * a.a_bs;
+	const long zw = a.w_sel ? a.w_sel[z] : z;
+	b.W = (const char *)a.W + zw * a.w_bs * WT::BYTES;
+	b.W2 = a.W2 ? (const char *)a.W2 + zw * a.w_bs * WT::BYTES : nullptr;
+	b.C = a.C + (long)z * a.c_bs;
+	b.bias = a.bias ? a.bias + (long)z * a.bias_bs : nullptr;
+	b.rows = a.rows ? a.rows + (long)z * a.rows_bs : nullptr;
+	b.M = a.counts ? a.counts[z] : a.M;
+	return b;
+}
+
+// ---- single tokens and short portions: one wave per output column streams its weight
+// row(s) once with 16-byte loads and keeps up to GEMV_MAX_M activation rows' sums.
+#define GEMV_MAX_M 8
+template <class WT, bool GLU>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_gemv_kernel(GemmArgs a) {
+	const GemmBatch b = gemm_batch<WT>(a, blockIdx.z);
+	const int lane = threadIdx.x & 63;
+	const int n = blockIdx.x * (SEQ_THREADS / 64) + (threadIdx.x >> 6);
+	if (n >= a.N || b.M <= 0)
+		return;
+	const int M = min(b.M, GEMV_MAX_M);
+	const float *ar[GEMV_MAX_M];
+	int crow[GEMV_MAX_M];
+#pragma unroll
+	for (int m = 0; m < GEMV_MAX_M; ++m) {
+		const int mm = min(m, M - 1);
+		const int s = b.rows ? b.rows[mm] : mm;
+		ar[m] = b.A + (size_t)(b.rows ? s / a.a_div : s) * a.lda;
+		crow[m] = (b.rows && !a.c_dense) ? s : mm;
+	}
+	float acc[GEMV_MAX_M] = {}, acc2[GEMV_MAX_M] = {};
+	const char *w = b.W + (size_t)n * a.ldw * WT::BYTES;
+	const char *w2 = GLU ? b.W2 + (size_t)n * a.ldw * WT::BYTES : nullptr;
+	constexpr int E = 8; // elements per lane and pass
+	const bool vec = (a.ldw % E == 0) && (((size_t)b.W | (size_t)(GLU ? b.W2 : b.W)) % 16 == 0) && (a.lda % 4 == 0) &&
+	                 ((size_t)b.A % 16 == 0);
+	for (int k0 = lane * E; k0 < a.K; k0 += 64 * E) {
+		float wf[E], wf2[E];
+		const bool full = vec && k0 + E <= a.K;
+		if (full) {
+			if constexpr (WT::BYTES == 2) {
+				WT::unpack(load16(w + (size_t)k0 * 2), wf);
+				if constexpr (GLU)
+					WT::unpack(load16(w2 + (size_t)k0 * 2), wf2);
+			} else {
+				WT::unpack(load16(w + (size_t)k0 * 4), wf);
+				WT::unpack(load16(w + (size_t)k0 * 4 + 16), wf + 4);
+				if constexpr (GLU) {
+					WT::unpack(load16(w2 + (size_t)k0 * 4), wf2);
+					WT::unpack(load16(w2 + (size_t)k0 * 4 + 16), wf2 + 4);
+				}
+			}
+		} else {
+#pragma unroll
+			for (int e = 0; e < E; ++e) {
+				wf[e] = k0 + e < a.K ? wload<WT>(w, k0 + e) : 0.0f;
+				if constexpr (GLU)
+					wf2[e] = k0 + e < a.K ? wload<WT>(w2, k0 + e) : 0.0f;
+			}
+		}
+#pragma unroll
+		for (int m = 0; m < GEMV_MAX_M; ++m) {
+			if (m < M) {
+				float x[E];
+				if (full) {
+					const float4_t x0 = *(const float4_t *)(ar[m] + k0), x1 = *(const float4_t *)(ar[m] + k0 + 4);
+#pragma unroll
+					for (int e = 0; e < 4; ++e) {
+						x[e] = x0[e];
+						x[4 + e] = x1[e];
+					}
+				} else {
+#pragma unroll
+					for (int e = 0; e < E; ++e)
+						x[e] = k0 + e < a.K ? ar[m][k0 + e] : 0.0f;
+				}
+#pragma unroll
+				for (int e = 0; e < E; ++e) {
+					acc[m] = fmaf(wf[e], x[e], acc[m]);
+					if constexpr (GLU)
+						acc2[m] = fmaf(wf2[e], x[e], acc2[m]);
+				}
+			}
+		}
+	}
+#pragma unroll
+	for (int m = 0; m < GEMV_MAX_M; ++m) {
+		if (m < M) {
+			const float v = wave_sum(acc[m]);
+			const float v2 = GLU ? wave_sum(acc2[m]) : 0.0f;
+			if (lane == 0)
+				b.C[(size_t)crow[m] * a.ldc + n] = epi_apply(a, v, v2, b.bias ? b.bias[n] : 0.0f);
+		}
+	}
+}
+
+// ---- portions: 64 x 64 output tiles, K in slabs of 32 through LDS.
+#define GT_BM 64
+#define GT_BN 64
+#define GT_BK 32
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+// WBF16: activations rounded to bf16 on the way into LDS; each of the 4 waves owns a
+// 32 x 32 quadrant as one v_mfma_f32_32x32x16_bf16 accumulator (A operand: lane l holds
+// row l & 31, k = 8 (l >> 5) .. + 7; C/D: column = lane & 31, row = (reg & 3) + 8 (reg >> 2)
+// + 4 (lane >> 5)). WF32: f32 FMA, each thread a 4 x 4 block.
+template <class WT, bool GLU>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_gemm_kernel(GemmArgs a) {
+	const GemmBatch b = gemm_batch<WT>(a, blockIdx.z);
+	const int m0 = blockIdx.y * GT_BM, n0 = blockIdx.x * GT_BN;
+	if (m0 >= b.M)
+		return;
+	const int tid = threadIdx.x;
+	__shared__ int arow[GT_BM], crow[GT_BM];
+	if (tid < GT_BM) {
+		const int m = m0 + tid;
+		int ra = -1, rc = -1;
+		if (m < b.M) {
+			const int s = b.rows ? b.rows[m] : m;
+			ra = b.rows ? s / a.a_div : s;
+			rc = (b.rows && !a.c_dense) ? s : m;
+		}
+		arow[tid] = ra;
+		crow[tid] = rc;
+	}
+	__syncthreads();
+
+	if constexpr (WT::BYTES == 2) {
+		constexpr int LD = GT_BK + 8; // bf16 elements per LDS row: 80 bytes, 16-byte aligned pieces
+		__shared__ __attribute__((aligned(16))) uint16_t As[GT_BM * LD], Bs[GT_BN * LD], Bs2[GLU ? GT_BN * LD : 8];
+		const int wave = tid >> 6, lane = tid & 63;
+		const int wm = (wave & 1) * 32, wn = (wave >> 1) * 32;
+		float16_t acc = {}, acc2 = {};
+		const int lr = tid >> 2, lk = (tid & 3) * 8; // loader: row, first k of 8
+		const int ra = arow[lr];
+		const int nb = n0 + lr;
+		const bool avec = a.lda % 4 == 0 && (size_t)b.A % 16 == 0;
+		const bool wvec = a.ldw % 8 == 0 && ((size_t)b.W | (size_t)(GLU ? b.W2 : b.W)) % 16 == 0;
+		for (int k0 = 0; k0 < a.K; k0 += GT_BK) {
+			const int k = k0 + lk;
+			u32x4_t pa = {0, 0, 0, 0}, pb = {0, 0, 0, 0}, pb2 = {0, 0, 0, 0};
+			if (ra >= 0) {
+				const float *src = b.A + (size_t)ra * a.lda + k;
+				float x[8];
+				if (avec && k + 8 <= a.K) {
+					const float4_t x0 = *(const float4_t *)src, x1 = *(const float4_t *)(src + 4);
+#pragma unroll
+					for (int e = 0; e < 4; ++e) {
+						x[e] = x0[e];
+						x[4 + e] = x1[e];
+					}
+				} else {
+#pragma unroll
+					for (int e = 0; e < 8; ++e)
+						x[e] = k + e < a.K ? src[e] : 0.0f;
+				}
+#pragma unroll
+				for (int e = 0; e < 4; ++e)
+					pa[e] = (uint32_t)f2bf(x[2 * e]) | ((uint32_t)f2bf(x[2 * e + 1]) << 16);
+			}
+			if (nb < a.N) {
+				const uint16_t *src = (const uint16_t *)b.W + (size_t)nb * a.ldw + k;
+				const uint16_t *src2 = GLU ? (const uint16_t *)b.W2 + (size_t)nb * a.ldw + k : nullptr;
+				if (wvec && k + 8 <= a.K) {
+					pb = load16(src);
+					if constexpr (GLU)
+						pb2 = load16(src2);
+				} else {
+#pragma unroll
+					for (int e = 0; e < 4; ++e) {
+						const uint32_t lo = k + 2 * e < a.K ? src[2 * e] : 0, hi = k + 2 * e + 1 < a.K ? src[2 * e + 1] : 0;
+						pb[e] = lo | (hi << 16);
+						if constexpr (GLU) {
+							const uint32_t lo2 = k + 2 * e < a.K ? src2[2 * e] : 0,
+							               hi2 = k + 2 * e + 1 < a.K ? src2[2 * e + 1] : 0;
+							pb2[e] = lo2 | (hi2 << 16);
+						}
+					}
+				}
+			}
+			__syncthreads(); // the previous slab's MFMAs have read LDS
+			*(u32x4_t *)(As + lr * LD + lk) = pa;
+			*(u32x4_t *)(Bs + lr * LD + lk) = pb;
+			if constexpr (GLU)
+				*(u32x4_t *)(Bs2 + lr * LD + lk) = pb2;
+			__syncthreads();
+#pragma unroll
+			for (int ks = 0; ks < GT_BK; ks += 16) {
+				const int kk = ks + 8 * (lane >> 5);
+				const bf16x8_t fa = __builtin_bit_cast(bf16x8_t, *(const u32x4_t *)(As + (wm + (lane & 31)) * LD + kk));
+				const bf16x8_t fb = __builtin_bit_cast(bf16x8_t, *(const u32x4_t *)(Bs + (wn + (lane & 31)) * LD + kk));
+				acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, acc, 0, 0, 0);
+				if constexpr (GLU) {
+					const bf16x8_t fb2 =
+					    __builtin_bit_cast(bf16x8_t, *(const u32x4_t *)(Bs2 + (wn + (lane & 31)) * LD + kk));
+					acc2 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb2, acc2, 0, 0, 0);
+				}
+			}
+		}
+		const int n = n0 + wn + (lane & 31);
+		if (n < a.N) {
+			const float bias = b.bias ? b.bias[n] : 0.0f;
+#pragma unroll
+			for (int r = 0; r < 16; ++r) {
+				const int ml = wm + (r & 3) + 8 * (r >> 2) + 4 * (lane >> 5);
+				const int rc = crow[ml];
+				if (rc >= 0)
+					b.C[(size_t)rc * a.ldc + n] = epi_apply(a, acc[r], GLU ? acc2[r] : 0.0f, bias);
+			}
+		}
+	} else {
+		constexpr int LDF = GT_BM + 4;
+		__shared__ float As[GT_BK * LDF], Bs[GT_BK * LDF], Bs2[GLU ? GT_BK * LDF : 4];
+		const int tx = tid & 15, ty = tid >> 4;
+		float acc[4][4] = {}, acc2[4][4] = {};
+		for (int k0 = 0; k0 < a.K; k0 += GT_BK) {
+			__syncthreads();
+			for (int idx = tid; idx < GT_BM * GT_BK; idx += SEQ_THREADS) {
+				const int r = idx / GT_BK, kk = idx % GT_BK;
+				const int k = k0 + kk;
+				const int ra = arow[r];
+				As[kk * LDF + r] = (ra >= 0 && k < a.K) ? b.A[(size_t)ra * a.lda + k] : 0.0f;
+				const int nb = n0 + r;
+				const bool ok = nb < a.N && k < a.K;
+				Bs[kk * LDF + r] = ok ? ((const float *)b.W)[(size_t)nb * a.ldw + k] : 0.0f;
+				if constexpr (GLU)
+					Bs2[kk * LDF + r] = ok ? ((const float *)b.W2)[(size_t)nb * a.ldw + k] : 0.0f;
+			}
+			__syncthreads();
+#pragma unroll 8
+			for (int kk = 0; kk < GT_BK; ++kk) {
+				const float4_t av = *(const float4_t *)(As + kk * LDF + ty * 4);
+				const float4_t bv = *(const float4_t *)(Bs + kk * LDF + tx * 4);
+				float4_t bv2 = {0, 0, 0, 0};
+				if constexpr (GLU)
+					bv2 = *(const float4_t *)(Bs2 + kk * LDF + tx * 4);
+#pragma unroll
+				for (int i = 0; i < 4; ++i)
+#pragma unroll
+					for (int j = 0; j < 4; ++j) {
+						acc[i][j] = fmaf(av[i], bv[j], acc[i][j]);
+						if constexpr (GLU)
+							acc2[i][j] = fmaf(av[i], bv2[j], acc2[i][j]);
+					}
+			}
+		}
+#pragma unroll
+		for (int i = 0; i < 4; ++i) {
+			const int rc = crow[ty * 4 + i];
+			if (rc < 0)
+				continue;
+#pragma unroll
+			for (int j = 0; j < 4; ++j) {
+				const int n = n0 + tx * 4 + j;
+				if (n < a.N)
+					b.C[(size_t)rc * a.ldc + n] =
+					    epi_apply(a, acc[i][j], GLU ? acc2[i][j] : 0.0f, b.bias ? b.bias[n] : 0.0f);
+			}
+		}
+	}
+}
+
+// ------------------------------------------------------------------ short causal convolution
+// out[t][c] = act(bias[c] + sum_j w[c][j] in(t - (taps - 1) + j)), in(tau) = Z[tau][col0 + c] for
+// tau >= 0, else the sequence's stored last inputs state[(taps - 1) + tau][c] (zeros at the start).
+__global__ __launch_bounds__(SEQ_THREADS) void seq_conv_kernel(const float *__restrict__ Z, int ldz, int col0, int C,
+                                                               int taps, const float *__restrict__ w,
+                                                               const float *__restrict__ bias, int silu,
+                                                               const float *__restrict__ state,
+                                                               float *__restrict__ out, int ldo, int T) {
+	const int c = blockIdx.x * SEQ_THREADS + threadIdx.x;
+	const int t = blockIdx.y;
+	if (c >= C)
+		return;
+	float acc = bias ? bias[c] : 0.0f;
+	for (int j = 0; j < taps; ++j) {
+		const int tau = t - (taps - 1) + j;
+		const float v = tau >= 0 ? Z[(size_t)tau * ldz + col0 + c] : state[(size_t)(taps - 1 + tau) * C + c];
+		acc = fmaf(w[(size_t)c * taps + j], v, acc);
+	}
+	out[(size_t)t * ldo + c] = silu ? sq_silu(acc) : acc;
+}
+// The stored inputs after a portion of T tokens: the last taps - 1 of (old state ++ Z rows).
+#define SEQ_MAX_TAPS 16
+__global__ __launch_bounds__(SEQ_THREADS) void seq_conv_state_kernel(const float *__restrict__ Z, int ldz, int col0,
+                                                                     int C, int taps, float *__restrict__ state,
+                                                                     int T) {
+	const int c = blockIdx.x * SEQ_THREADS + threadIdx.x;
+	if (c >= C)
+		return;
+	float keep[SEQ_MAX_TAPS];
+#pragma unroll
+	for (int i = 0; i < SEQ_MAX_TAPS; ++i) {
+		if (i < taps - 1) {
+			const int tau = T - (taps - 1) + i;
+			keep[i] = tau >= 0 ? Z[(size_t)tau * ldz + col0 + c] : state[(size_t)(taps - 1 + tau) * C + c];
+		}
+	}
+#pragma unroll
+	for (int i = 0; i < SEQ_MAX_TAPS; ++i)
+		if (i < taps - 1)
+			state[(size_t)i * C + c] = keep[i];
+}
+
+// ------------------------------------------------------------------ real-gated linear recurrence
+// Per channel, over the portion's tokens in order: log a = -8 r softplus(lam), a = exp(log a),
+// S = a S + sqrt(1 - a^2) (i u); out = S * gelu_tanh(gate branch). 1 - a^2 is taken as
+// -expm1(2 log a), which keeps its relative precision when a is close to 1.
+__global__ __launch_bounds__(SEQ_THREADS) void seq_rglru_scan_kernel(const float *__restrict__ R,
+                                                                     const float *__restrict__ I,
+                                                                     const float *__restrict__ U, int W,
+                                                                     const float *__restrict__ Z, int ldz,
+                                                                     const float *__restrict__ lam,
+                                                                     float *__restrict__ state, float *__restrict__ out,
+                                                                     int T) {
+	const int c = blockIdx.x * SEQ_THREADS + threadIdx.x;
+	if (c >= W)
+		return;
+	const float sp = sq_softplus(lam[c]);
+	float S = state[c];
+#pragma unroll 4
+	for (int t = 0; t < T; ++t) {
+		const size_t o = (size_t)t * W + c;
+		const float la = -8.0f * R[o] * sp;
+		const float aa = expf(la);
+		const float mult = sqrtf(-expm1f(2.0f * la));
+		S = fmaf(aa, S, mult * (I[o] * U[o]));
+		out[o] = S * sq_gelu_tanh(Z[(size_t)t * ldz + c]);
+	}
+	state[c] = S;
+}
+
+// ------------------------------------------------------------------ gated delta rule
+// After the convolutions: q and k to unit length per head (q also x dim^-1/2), beta =
+// sigmoid, decay g = exp(-exp(a_log) softplus(a + dt_bias)). QKV: [T][ldq] = q | k | v
+// (convolved, silu); Z columns bcol.. = beta logits, acol.. = decay inputs. One workgroup per token.
+__global__ __launch_bounds__(SEQ_THREADS) void seq_delta_prep_kernel(float *__restrict__ QKV, int ldq, int KH, int D,
+                                                                     const float *__restrict__ Z, int ldz, int bcol,
+                                                                     int acol, int H, const float *__restrict__ a_log,
+                                                                     const float *__restrict__ dt_bias,
+                                                                     float *__restrict__ BG) {
+	const int t = blockIdx.x;
+	const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+	float *row = QKV + (size_t)t * ldq;
+	const float qs = 1.0f / sqrtf((float)D);
+	for (int seg = wave; seg < 2 * KH; seg += SEQ_THREADS / 64) {
+		float *x = row + (size_t)seg * D;
+		float ss = 0.0f;
+		for (int i = lane; i < D; i += 64)
+			ss = fmaf(x[i], x[i], ss);
+		ss = wave_sum(ss);
+		const float r = (1.0f / sqrtf(ss + 1e-6f)) * (seg < KH ? qs : 1.0f);
+		for (int i = lane; i < D; i += 64)
+			x[i] *= r;
+	}
+	for (int h = threadIdx.x; h < H; h += SEQ_THREADS) {
+		BG[(size_t)t * 2 * H + h] = sq_sigmoid(Z[(size_t)t * ldz + bcol + h]);
+		BG[(size_t)t * 2 * H + H + h] =
+		    expf(-expf(a_log[h]) * sq_softplus(Z[(size_t)t * ldz + acol + h] + dt_bias[h]));
+	}
+}
+
+__device__ __forceinline__ float sum8(float v) { // over aligned groups of 8 lanes
+	v += dpp<0xB1>(v);
+	v += dpp<0x4E>(v);
+	v += dpp<0x141>(v);
+	return v;
+}
+
+// The recurrence itself. The columns of a head's [dim][vdim] state never mix, so one group
+// of 8 lanes owns one column (its dim entries interleaved over the lanes, R per lane, in
+// registers) and walks the portion's tokens in order:
+//   S *= g;  u = beta (v - S.k);  S += k u;  o = S.q
+// (the read-out after the write). The next token's operands are loaded while the current
+// one is applied. grid (ceil(vdim / 32), heads).
+template <int R>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__restrict__ QKV, int ldq, int KH, int D,
+                                                                int H, int V, const float *__restrict__ BG,
+                                                                float *__restrict__ state, float *__restrict__ O,
+                                                                int T) {
+	const int h = blockIdx.y, kh = h / (H / KH);
+	const int col = blockIdx.x * (SEQ_THREADS / 8) + (threadIdx.x >> 3), sub = threadIdx.x & 7;
+	const bool live = col < V;
+	const int vc = live ? col : V - 1;
+	float S[R];
+	float *sp = state + (size_t)h * D * V;
+#pragma unroll
+	for (int i = 0; i < R; ++i) {
+		const int d = sub + 8 * i;
+		S[i] = (d < D) ? sp[(size_t)d * V + vc] : 0.0f;
+	}
+	const int qo = kh * D, ko = KH * D + kh * D, vo = 2 * KH * D + h * V + vc;
+	float kn[R], qn[R], vn, bn, gn;
+	auto load = [&](int t) {
+		const float *row = QKV + (size_t)t * ldq;
+#pragma unroll
+		for (int i = 0; i < R; ++i) {
+			const int d = sub + 8 * i;
+			kn[i] = d < D ? row[ko + d] : 0.0f;
+			qn[i] = d < D ? row[qo + d] : 0.0f;
+		}
+		vn = row[vo];
+		bn = BG[(size_t)t * 2 * H + h];
+		gn = BG[(size_t)t * 2 * H + H + h];
+	};
+	load(0);
+	for (int t = 0; t < T; ++t) {
+		float k[R], q[R];
+#pragma unroll
+		for (int i = 0; i < R; ++i) {
+			k[i] = kn[i];
+			q[i] = qn[i];
+		}
+		const float v = vn, beta = bn, g = gn;
+		if (t + 1 < T)
+			load(t + 1);
+		float d0 = 0.0f, d1 = 0.0f;
+#pragma unroll
+		for (int i = 0; i < R; ++i) {
+			S[i] *= g;
+			if (i & 1)
+				d1 = fmaf(S[i], k[i], d1);
+			else
+				d0 = fmaf(S[i], k[i], d0);
+		}
+		const float u = beta * (v - sum8(d0 + d1));
+		float o0 = 0.0f, o1 = 0.0f;
+#pragma unroll
+		for (int i = 0; i < R; ++i) {
+			S[i] = fmaf(k[i], u, S[i]);
+			if (i & 1)
+				o1 = fmaf(S[i], q[i], o1);
+			else
+				o0 = fmaf(S[i], q[i], o0);
+		}
+		const float o = sum8(o0 + o1);
+		if (sub == 0 && live)
+			O[(size_t)t * H * V + h * V + col] = o;
+	}
+	if (live) {
+#pragma unroll
+		for (int i = 0; i < R; ++i) {
+			const int d = sub + 8 * i;
+			if (d < D)
+				sp[(size_t)d * V + col] = S[i];
+		}
+	}
+}
+
+// Each head's read-out divided by its root mean square over vdim, times the shared weight,
+// times silu of the output gate (Z columns gcol..). One workgroup per token, a wave per head.
+__global__ __launch_bounds__(SEQ_THREADS) void seq_delta_out_kernel(const float *__restrict__ O, int H, int V,
+                                                                    const float *__restrict__ w, float eps,
+                                                                    const float *__restrict__ Z, int ldz, int gcol,
+                                                                    float *__restrict__ out) {
+	const int t = blockIdx.x;
+	const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+	for (int h = wave; h < H; h += SEQ_THREADS / 64) {
+		const float *o = O + (size_t)t * H * V + (size_t)h * V;
+		float ss = 0.0f;
+		for (int i = lane; i < V; i += 64)
+			ss = fmaf(o[i], o[i], ss);
+		ss = wave_sum(ss);
+		const float r = 1.0f / sqrtf(ss / (float)V + eps);
+		for (int i = lane; i < V; i += 64)
+			out[(size_t)t * H * V + (size_t)h * V + i] =
+			    o[i] * r * w[i] * sq_silu(Z[(size_t)t * ldz + gcol + h * V + i]);
+	}
+}
+
+// ------------------------------------------------------------------ latent attention
+// Attention over the cached latent itself: with q~ = W_uk[h]^T q (per head, a kv_rank
+// vector) the score q . (W_uk[h] c_j) equals q~ . c_j, and sum_j p_j (W_uv[h] c_j) equals
+// W_uv[h] (sum_j p_j c_j); so every head of a token reads the same cached rows, as in
+// multi-query attention with key = value = c. Rows r = t * H + h of Qa / Ctx; row r sees
+// cache rows j <= st->pos + r / H. Scores, softmax (running maximum and sum per row) and the
+// weighted sums are f32. A workgroup owns ATT_BR rows and walks the keys in tiles of 64:
+// each wave scores 4 rows x 64 keys (a lane per key), then every thread updates NACC
+// (row, latent entry) sums. Dynamic LDS: att_lds_bytes(rank).
+#define ATT_BR 16
+#define ATT_KT 64
+template <class CT, int NACC>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_latent_attn_kernel(const float *__restrict__ Qa,
+                                                                      const CT *__restrict__ cache, int rank, int H,
+                                                                      int NR, float scale,
+                                                                      const StepState *__restrict__ st,
+                                                                      float *__restrict__ Ctx) {
+	extern __shared__ float lds[];
+	const int ldc = rank + 1;
+	float *qs = lds;                      // [ATT_BR][rank]
+	float *cs = qs + ATT_BR * rank;       // [ATT_KT][rank + 1]
+	float *ps = cs + ATT_KT * ldc;        // [ATT_BR][ATT_KT]
+	float *alpha = ps + ATT_BR * ATT_KT;  // [ATT_BR]
+	float *lsum = alpha + ATT_BR;         // [ATT_BR]
+	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+	const int r0 = blockIdx.x * ATT_BR;
+	const int pos0 = st->pos;
+	const int rlast = min(r0 + ATT_BR, NR) - 1;
+	const int kmax = pos0 + rlast / H; // the last visible key of the workgroup's last row
+	for (int i = tid; i < ATT_BR * rank; i += SEQ_THREADS) {
+		const int r = r0 + i / rank;
+		qs[i] = r < NR ? Qa[(size_t)r * rank + i % rank] * scale : 0.0f;
+	}
+	float acc[NACC] = {};
+	float mrun[4], lrun[4];
+	int lim[4];
+#pragma unroll
+	for (int i = 0; i < 4; ++i) {
+		const int r = r0 + wave * 4 + i;
+		mrun[i] = -FLT_MAX;
+		lrun[i] = 0.0f;
+		lim[i] = r < NR ? pos0 + r / H : -1;
+	}
+	for (int kt = 0; kt <= kmax; kt += ATT_KT) {
+		__syncthreads(); // the previous tile's sums have read cs / ps
+		for (int i = tid; i < ATT_KT * rank; i += SEQ_THREADS) {
+			const int j = kt + i / rank, d = i % rank;
+			float v = 0.0f;
+			if (j <= kmax) {
+				if constexpr (sizeof(CT) == 2)
+					v = bf2f(cache[(size_t)j * rank + d]);
+				else
+					v = cache[(size_t)j * rank + d];
+			}
+			cs[(i / rank) * ldc + d] = v;
+		}
+		__syncthreads();
+		{
+			float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+			const float *cj = cs + lane * ldc;
+			const float *q0 = qs + (wave * 4) * rank;
+			for (int d = 0; d < rank; ++d) {
+				const float c = cj[d];
+#pragma unroll
+				for (int i = 0; i < 4; ++i)
+					s[i] = fmaf(q0[i * rank + d], c, s[i]);
+			}
+#pragma unroll
+			for (int i = 0; i < 4; ++i) {
+				const bool vis = kt + lane <= lim[i];
+				const float sv = vis ? s[i] : -FLT_MAX;
+				const float mx = wave_max(sv);
+				const float mnew = fmaxf(mrun[i], mx);
+				const float p = vis ? expf(sv - mnew) : 0.0f;
+				const float al = expf(mrun[i] - mnew); // 1 when nothing is visible yet, 0 after the first key
+				lrun[i] = lrun[i] * al + wave_sum(p);
+				mrun[i] = mnew;
+				ps[(wave * 4 + i) * ATT_KT + lane] = p;
+				if (lane == 0)
+					alpha[wave * 4 + i] = al;
+			}
+		}
+		__syncthreads();
+#pragma unroll
+		for (int a = 0; a < NACC; ++a) {
+			const int idx = tid + a * SEQ_THREADS;
+			if (idx < ATT_BR * rank) {
+				const int r = idx / rank, d = idx % rank;
+				float v = acc[a] * alpha[r];
+				const float *pr = ps + r * ATT_KT;
+#pragma unroll 8
+				for (int j = 0; j < ATT_KT; ++j)
+					v = fmaf(pr[j], cs[j * ldc + d], v);
+				acc[a] = v;
+			}
+		}
+	}
+	if (lane == 0) {
+#pragma unroll
+		for (int i = 0; i < 4; ++i)
+			lsum[wave * 4 + i] = lrun[i];
+	}
+	__syncthreads();
+#pragma unroll
+	for (int a = 0; a < NACC; ++a) {
+		const int idx = tid + a * SEQ_THREADS;
+		if (idx < ATT_BR * rank) {
+			const int r = idx / rank, d = idx % rank;
+			if (r0 + r < NR)
+				Ctx[(size_t)(r0 + r) * rank + d] = acc[a] / lsum[r];
+		}
+	}
+}
+static inline size_t att_lds_bytes(int rank) {
+	return sizeof(float) * ((size_t)ATT_BR * rank + (size_t)ATT_KT * (rank + 1) + ATT_BR * ATT_KT + 2 * ATT_BR);
+}
+
+// ------------------------------------------------------------------ routed experts
+// One workgroup per token: router logits in f32, softmax over all experts, a group's score
+// = its best expert's, only experts of the `keep` best groups can be chosen, the `top`
+// largest scores among them win (ties: the lower index); weight = score * rscale, not
+// renormalised. Also the shared expert's gate sigmoid(w_sg . h). Dynamic LDS: E floats.
+#define SEQ_MAX_GROUPS 64
+__global__ __launch_bounds__(SEQ_THREADS) void seq_router_kernel(const float *__restrict__ Hn, int width,
+                                                                 const float *__restrict__ Wr, int E, int top, int G,
+                                                                 int keep, float rscale,
+                                                                 const float *__restrict__ w_sg, int *__restrict__ idx,
+                                                                 float *__restrict__ wt, float *__restrict__ sgate) {
+	extern __shared__ float sc[];
+	const int t = blockIdx.x;
+	const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+	const float *h = Hn + (size_t)t * width;
+	for (int e = wave; e < E + (w_sg ? 1 : 0); e += SEQ_THREADS / 64) {
+		const float *w = e < E ? Wr + (size_t)e * width : w_sg;
+		float a = 0.0f;
+		for (int i = lane; i < width; i += 64)
+			a = fmaf(w[i], h[i], a);
+		a = wave_sum(a);
+		if (lane == 0) {
+			if (e < E)
+				sc[e] = a;
+			else
+				sgate[t] = sq_sigmoid(a);
+		}
+	}
+	__syncthreads();
+	if (threadIdx.x != 0)
+		return;
+	float mx = -FLT_MAX;
+	for (int e = 0; e < E; ++e)
+		mx = fmaxf(mx, sc[e]);
+	float sum = 0.0f;
+	for (int e = 0; e < E; ++e) {
+		sc[e] = expf(sc[e] - mx);
+		sum += sc[e];
+	}
+	const float inv = 1.0f / sum;
+	const int gs = E / G;
+	unsigned long long allowed = 0ull; // groups that may be chosen from (G <= 64)
+	float gsc[SEQ_MAX_GROUPS];
+	for (int g = 0; g < G; ++g) {
+		float m = -1.0f;
+		for (int e = g * gs; e < (g + 1) * gs; ++e)
+			m = fmaxf(m, sc[e]);
+		gsc[g] = m;
+	}
+	for (int k = 0; k < keep; ++k) {
+		int best = -1;
+		float bv = -2.0f;
+		for (int g = 0; g < G; ++g)
+			if (!((allowed >> g) & 1ull) && gsc[g] > bv) {
+				bv = gsc[g];
+				best = g;
+			}
+		allowed |= 1ull << best;
+	}
+	for (int k = 0; k < top; ++k) {
+		int best = 0;
+		float bv = -1.0f;
+		for (int e = 0; e < E; ++e)
+			if (((allowed >> (e / gs)) & 1ull) && sc[e] > bv) {
+				bv = sc[e];
+				best = e;
+			}
+		idx[(size_t)t * top + k] = best;
+		wt[(size_t)t * top + k] = bv * inv * rscale;
+		sc[best] = -1.0f; // taken
+	}
+}
+
+// Slot s = t * top + k goes onto its expert's list (any order: every slot's rows are
+// computed independently of their neighbours in the list).
+__global__ __launch_bounds__(SEQ_THREADS) void seq_moe_lists_kernel(const int *__restrict__ idx, int n_slots,
+                                                                    int *__restrict__ counts, int *__restrict__ lists,
+                                                                    int cap) {
+	const int s = blockIdx.x * SEQ_THREADS + threadIdx.x;
+	if (s >= n_slots)
+		return;
+	const int e = idx[s];
+	const int p = atomicAdd(&counts[e], 1);
+	lists[(size_t)e * cap + p] = s;
+}
+__global__ void seq_fill_int_kernel(int *p, int n, int v) {
+	const int i = blockIdx.x * blockDim.x + threadIdx.x;
+	if (i < n)
+		p[i] = v;
+}
+__global__ void seq_fill_float_kernel(float *p, size_t n, float v) {
+	for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+		p[i] = v;
+}
+
+// Y[t] = sum_k wt[t][k] Yx[t * top + k] (+ sgate[t] * Ys[t]).
+__global__ __launch_bounds__(SEQ_THREADS) void seq_moe_combine_kernel(const float *__restrict__ Yx,
+                                                                      const float *__restrict__ wt, int top,
+                                                                      const float *__restrict__ Ys,
+                                                                      const float *__restrict__ sgate, int width,
+                                                                      float *__restrict__ Y) {
+	const int t = blockIdx.y;
+	const int n = blockIdx.x * SEQ_THREADS + threadIdx.x;
+	if (n >= width)
+		return;
+	float v = 0.0f;
+	for (int k = 0; k < top; ++k)
+		v = fmaf(wt[(size_t)t * top + k], Yx[((size_t)t * top + k) * width + n], v);
+	if (Ys)
+		v = fmaf(sgate[t], Ys[(size_t)t * width + n], v);
+	Y[(size_t)t * width + n] = v;
+}

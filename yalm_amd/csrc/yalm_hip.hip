@@ -23,98 +23,6 @@
 #include "gemv.h"
 #include "misc_kernels.h"
 
-// ------------------------------------------------------------------ errors
-static thread_local std::string g_err;
-
-void set_err(const std::string &s) {
-	g_err = s;
-}
-
-extern "C" const char *yalm_last_error(void) {
-	return g_err.c_str();
-}
-
-// ------------------------------------------------------------------ shim
-extern "C" int yalm_set_device(int device) {
-	HIPCHK(hipSetDevice(device));
-	return YALM_OK;
-}
-
-extern "C" void *yalm_upload(const void *host, size_t size) {
-	void *dev = nullptr;
-	if (hipMalloc(&dev, size ? size : 1) != hipSuccess) {
-		set_err("hipMalloc failed in yalm_upload");
-		return nullptr;
-	}
-	if (size && hipMemcpy(dev, host, size, hipMemcpyHostToDevice) != hipSuccess) {
-		set_err("hipMemcpy H2D failed in yalm_upload");
-		(void)hipFree(dev);
-		return nullptr;
-	}
-	return dev;
-}
-
-extern "C" void *yalm_alloc(size_t size) {
-	void *dev = nullptr;
-	if (hipMalloc(&dev, size ? size : 1) != hipSuccess) {
-		set_err("hipMalloc failed in yalm_alloc");
-		return nullptr;
-	}
-	if (hipMemset(dev, 0, size ? size : 1) != hipSuccess) {
-		set_err("hipMemset failed in yalm_alloc");
-		(void)hipFree(dev);
-		return nullptr;
-	}
-	return dev;
-}
-
-extern "C" int yalm_download(void *host, const void *device, size_t size) {
-	HIPCHK(hipMemcpy(host, device, size, hipMemcpyDeviceToHost));
-	return YALM_OK;
-}
-
-extern "C" int yalm_register_host(void *host, size_t size) {
-	HIPCHK(hipHostRegister(host, size, hipHostRegisterDefault));
-	return YALM_OK;
-}
-
-extern "C" int yalm_unregister_host(void *host) {
-	HIPCHK(hipHostUnregister(host));
-	return YALM_OK;
-}
-
-extern "C" int yalm_free(void *device) {
-	HIPCHK(hipFree(device));
-	return YALM_OK;
-}
-
-extern "C" int yalm_stream_create(yalm_stream *out) {
-	ARGCHK(out, "null stream out");
-	hipStream_t s;
-	HIPCHK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
-	*out = reinterpret_cast<yalm_stream>(s);
-	return YALM_OK;
-}
-
-// A stream restricted to CU block `part` of `n_parts` (hipExtStreamCreateWithCUMask):
-// bits [part * ncu / n_parts, (part + 1) * ncu / n_parts). The driver spreads such a block
-// evenly over the 8 XCDs (tools/cumask_probe.hip, profiles/r6a_cumask_probe.txt: 256 / N CUs
-// on all 8 XCCs, disjoint between parts); an interleaved mask (bit i to part i mod N) was
-// not honoured (every part ran on all 256 CUs). Used to run N tensor-parallel rank
-// processes on ONE GPU as N disjoint sets of CUs (the multi-GPU rehearsal).
-extern "C" int yalm_stream_create_cu_part(int part, int n_parts, yalm_stream *out) {
-	ARGCHK(out && n_parts >= 1 && part >= 0 && part < n_parts, "yalm_stream_create_cu_part: bad argument");
-	const int ncu = device_cu_count();
-	ARGCHK(ncu % n_parts == 0 && ncu <= 32 * YALM_CU_MASK_WORDS, "yalm_stream_create_cu_part: CUs do not divide");
-	uint32_t m[YALM_CU_MASK_WORDS] = {};
-	for (int i = part * (ncu / n_parts); i < (part + 1) * (ncu / n_parts); ++i)
-		m[i / 32] |= 1u << (i % 32);
-	hipStream_t s;
-	HIPCHK(hipExtStreamCreateWithCUMask(&s, (uint32_t)((ncu + 31) / 32), m));
-	*out = reinterpret_cast<yalm_stream>(s);
-	return YALM_OK;
-}
-
 // The CUs a stream may run on (all of them for an ordinary stream).
 static int stream_cu_mask(hipStream_t s, uint32_t *m) {
 	const int ncu = device_cu_count();
@@ -128,36 +36,7 @@ static int stream_cu_mask(hipStream_t s, uint32_t *m) {
 	return YALM_OK;
 }
 
-extern "C" int yalm_stream_destroy(yalm_stream s) {
-	HIPCHK(hipStreamDestroy(reinterpret_cast<hipStream_t>(s)));
-	return YALM_OK;
-}
-
-extern "C" int yalm_stream_sync(yalm_stream s) {
-	HIPCHK(hipStreamSynchronize(reinterpret_cast<hipStream_t>(s)));
-	return YALM_OK;
-}
-
-extern "C" int yalm_synth(void *device, size_t n, int dtype, uint64_t seed, float scale, float offset, yalm_stream s) {
-	ARGCHK(dtype == YALM_F32 || dtype == YALM_F16 || dtype == YALM_F8E5M2, "yalm_synth: bad dtype");
-	hipStream_t st = reinterpret_cast<hipStream_t>(s);
-	synth_kernel<<<4096, 256, 0, st>>>(device, n, dtype, seed, scale, offset);
-	HIPCHK(hipGetLastError());
-	return YALM_OK;
-}
-
 // ------------------------------------------------------------------ launch helpers
-int device_cu_count() {
-	static int n = 0;
-	if (!n) {
-		int dev = 0;
-		if (hipGetDevice(&dev) != hipSuccess ||
-		    hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-			n = 256;
-	}
-	return n;
-}
-
 // Row-block geometry (gemv_rb_kernel): `gpw` = workgroups per CU (default 1),
 // threads 512 (8 waves), U = 8 loads in flight per wave.
 // whole-row mode (gemv.h ROWS): W1|W3 (PGlu), W2 / Wo (PResidual), QKV (PQKV) when the rows divide

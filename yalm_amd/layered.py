@@ -1,0 +1,346 @@
+"""Layer-list model designs: configuration, checkpoint reading and weight packing.
+
+A layer-list design gives every layer its own token mixer and feed-forward
+(include/yalm_hip.h, "layer-list models"). ``LayeredConfig`` is the engine-facing
+description; a design registers a reader that turns its ``config.json`` into one and
+a packer that turns its checkpoint tensors into the engine's per-layer tensors
+(concatenated input projections, per-head transposed key up-projections, stacked
+experts). ``Sinulorn`` is the first such design.
+
+Checkpoints are folders with ``config.json`` and ``model.safetensors`` (bf16
+matrices; read with yalmfile.read_yalm, the same container the .yalm files use).
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import json
+import os
+
+import numpy as np
+
+from . import models as M
+
+MIX_LATENT, MIX_RGLRU, MIX_DELTA = 0, 1, 2
+FF_NONE, FF_DENSE, FF_MOE = 0, 1, 2
+
+
+@dataclasses.dataclass
+class LayerSpec:
+    mixer: int
+    heads: int = 0
+    kv_heads: int = 0
+    dim: int = 0
+    vdim: int = 0
+    kv_rank: int = 0
+    q_rank: int = 0
+    kv_from: int = -1
+    attn_scale: float = 0.0
+    rec_width: int = 0
+    blocks: int = 0
+    conv: int = 0
+    ff_kind: int = FF_NONE
+    ff: int = 0
+    experts: int = 0
+    top: int = 0
+    groups: int = 1
+    groups_keep: int = 1
+    router_scale: float = 1.0
+    limit: float = 0.0
+    shared_ff: int = 0
+    shared_limit: float = 0.0
+
+    @property
+    def in_rows(self) -> int:
+        """Rows of the concatenated input projection w_in."""
+        if self.mixer == MIX_LATENT:
+            return self.q_rank + (self.kv_rank if self.kv_from < 0 else 0)
+        if self.mixer == MIX_RGLRU:
+            return 2 * self.rec_width
+        return 2 * self.kv_heads * self.dim + 2 * self.heads * self.vdim + 2 * self.heads
+
+    @property
+    def mix_out(self) -> int:
+        """Columns of the mixer's output projection."""
+        return self.rec_width if self.mixer == MIX_RGLRU else self.heads * self.vdim
+
+
+@dataclasses.dataclass
+class LayeredConfig:
+    arch: str
+    width: int
+    vocab: int
+    layers: list
+    embed_scale: float = 1.0
+    norm_eps: float = 1e-5
+    max_tokens: int = 4096
+    weight_dtype: int = M.BF16
+
+    def with_(self, **kw) -> "LayeredConfig":
+        return dataclasses.replace(self, **kw)
+
+
+def packed_shapes(c: LayeredConfig, l: LayerSpec) -> dict:
+    """field -> (shape, kind) of one layer's engine tensors; kind "w": a matrix of the
+    model's weight dtype, "f": f32."""
+    W = c.width
+    out = {"norm1": ((W,), "f"), "norm1b": ((W,), "f")}
+    if l.ff_kind != FF_NONE:
+        out.update(norm2=((W,), "f"), norm2b=((W,), "f"))
+    out["w_in"] = ((l.in_rows, W), "w")
+    out["w_o"] = ((W, l.mix_out), "w")
+    if l.mixer == MIX_LATENT:
+        out["q_norm"] = ((l.q_rank,), "f")
+        if l.kv_from < 0:
+            out["kv_norm"] = ((l.kv_rank,), "f")
+        out["w_uq"] = ((l.heads * l.dim, l.q_rank), "w")
+        out["w_ukt"] = ((l.heads, l.kv_rank, l.dim), "w")
+        out["w_uv"] = ((l.heads * l.vdim, l.kv_rank), "w")
+    elif l.mixer == MIX_RGLRU:
+        bs = l.rec_width // l.blocks
+        out.update(
+            in_bias=((2 * l.rec_width,), "f"), conv_w=((l.rec_width, l.conv), "f"), conv_b=((l.rec_width,), "f"),
+            gate_a=((l.blocks, bs, bs), "f"), gate_a_b=((l.rec_width,), "f"),
+            gate_i=((l.blocks, bs, bs), "f"), gate_i_b=((l.rec_width,), "f"), lam=((l.rec_width,), "f"),
+        )
+    else:
+        cc = 2 * l.kv_heads * l.dim + l.heads * l.vdim
+        out.update(conv_w=((cc, l.conv), "f"), a_log=((l.heads,), "f"), dt_bias=((l.heads,), "f"),
+                   out_norm=((l.vdim,), "f"))
+    if l.ff_kind == FF_DENSE:
+        out.update(w_gate=((l.ff, W), "w"), w_up=((l.ff, W), "w"), w_down=((W, l.ff), "w"))
+    elif l.ff_kind == FF_MOE:
+        out.update(router=((l.experts, W), "f"), w_gate=((l.experts, l.ff, W), "w"),
+                   w_up=((l.experts, l.ff, W), "w"), w_down=((l.experts, W, l.ff), "w"))
+        if l.shared_ff:
+            out.update(shared_sg=((W,), "f"), ws_gate=((l.shared_ff, W), "w"), ws_up=((l.shared_ff, W), "w"),
+                       ws_down=((W, l.shared_ff), "w"))
+    return out
+
+
+# ------------------------------------------------------------------ bf16 <-> f32 on the host
+def bf16_to_f32(bits: np.ndarray) -> np.ndarray:
+    return (np.asarray(bits, np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def f32_to_bf16(x: np.ndarray) -> np.ndarray:
+    """Round to nearest even on the f32 bits."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def _as_f32(a: np.ndarray) -> np.ndarray:
+    return bf16_to_f32(a) if a.dtype == np.uint16 else np.asarray(a, np.float32)
+
+
+def _as_weight(a: np.ndarray, dtype: int) -> np.ndarray:
+    """A matrix in the engine's storage: bf16 bits (uint16) or f32."""
+    if dtype == M.F32:
+        return np.ascontiguousarray(_as_f32(a))
+    if dtype != M.BF16:
+        raise ValueError("layer-list models run with bf16 or f32 matrices")
+    return np.ascontiguousarray(a if a.dtype == np.uint16 else f32_to_bf16(a))
+
+
+# ------------------------------------------------------------------ Sinulorn
+SINULORN_MIXERS = {"latent_attention": MIX_LATENT, "rglru": MIX_RGLRU, "delta": MIX_DELTA}
+
+
+def sinulorn_config(cfg: dict, max_tokens: int = 4096, weight_dtype: int = M.BF16) -> LayeredConfig:
+    """config.json of a Sinulorn checkpoint -> LayeredConfig. Every size and every
+    constant that can differ between models of the design is read from cfg."""
+    layers = []
+    for e in cfg["layers"]:
+        m = e["mixer"]
+        kind = SINULORN_MIXERS.get(e["type"])
+        if kind is None:
+            raise ValueError(f"unknown mixer type {e['type']!r}")
+        if kind == MIX_LATENT:
+            s = LayerSpec(kind, heads=m["heads"], dim=m["dim"], vdim=m["vdim"], kv_rank=m["kv_rank"],
+                          q_rank=m["q_rank"], kv_from=m.get("kv_from", -1) if m.get("kv_from") is not None else -1,
+                          attn_scale=float(m["scale"]))
+        elif kind == MIX_RGLRU:
+            s = LayerSpec(kind, rec_width=m["width"], blocks=m["blocks"], conv=m["conv"])
+        else:
+            s = LayerSpec(kind, heads=m["heads"], kv_heads=m["kv_heads"], dim=m["dim"], vdim=m["vdim"], conv=m["conv"])
+        mlp = e.get("mlp")
+        if mlp:
+            if mlp["kind"] == "dense":
+                s.ff_kind, s.ff = FF_DENSE, mlp["ff"]
+            elif mlp["kind"] == "moe":
+                r = mlp["router"]
+                g = r.get("groups") or {"count": 1, "keep": 1}
+                s.ff_kind, s.ff, s.limit = FF_MOE, mlp["expert"]["ff"], float(mlp["expert"]["limit"])
+                s.experts, s.top, s.router_scale = r["experts"], r["top"], float(r.get("scale", 1.0))
+                s.groups, s.groups_keep = g["count"], g["keep"]
+                sh = mlp.get("shared")
+                if sh:
+                    s.shared_ff, s.shared_limit = sh["ff"], float(sh["limit"])
+            else:
+                raise ValueError(f"unknown feed-forward kind {mlp['kind']!r}")
+        layers.append(s)
+    return LayeredConfig(
+        arch="Sinulorn", width=cfg["width"], vocab=cfg["vocab"], layers=layers,
+        embed_scale=float(cfg["embedding"]["scale"]), norm_eps=float(cfg["norm"]["eps"]),
+        max_tokens=max_tokens, weight_dtype=weight_dtype,
+    )
+
+
+def sinulorn_tensor_shapes(cfg: dict) -> dict:
+    """Checkpoint tensor name -> shape for a Sinulorn config.json."""
+    W = cfg["width"]
+    out = {"embed": (cfg["vocab"], W), "final.norm": (W,), "head": (cfg["vocab"], W)}
+    for i, e in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", e["mixer"]
+        out[p + "norm1"] = out[p + "norm1b"] = (W,)
+        x = p + "mix."
+        if e["type"] == "latent_attention":
+            H, D, V = m["heads"], m["dim"], m["vdim"]
+            out[x + "dq"], out[x + "dq.norm"], out[x + "uq"] = (m["q_rank"], W), (m["q_rank"],), (H * D, m["q_rank"])
+            if m.get("kv_from") is None:
+                out[x + "dkv"], out[x + "dkv.norm"] = (m["kv_rank"], W), (m["kv_rank"],)
+            out[x + "uk"], out[x + "uv"], out[x + "o"] = (H * D, m["kv_rank"]), (H * V, m["kv_rank"]), (W, H * V)
+        elif e["type"] == "rglru":
+            R, B = m["width"], m["blocks"]
+            for n in ("y", "x"):
+                out[x + n], out[x + n + ".b"] = (R, W), (R,)
+            out[x + "conv"], out[x + "conv.b"] = (R, m["conv"]), (R,)
+            for n in ("ra", "ri"):
+                out[x + n], out[x + n + ".b"] = (B, R // B, R // B), (B, R // B)
+            out[x + "lam"], out[x + "o"] = (R,), (W, R)
+        else:
+            H, KH, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            for n, rows in (("q", KH * D), ("k", KH * D), ("v", H * V)):
+                out[x + n], out[x + n + ".conv"] = (rows, W), (rows, m["conv"])
+            out[x + "b"] = out[x + "a"] = (H, W)
+            out[x + "A_log"] = out[x + "dt_bias"] = (H,)
+            out[x + "norm"], out[x + "g"], out[x + "o"] = (V,), (H * V, W), (W, H * V)
+        mlp = e.get("mlp")
+        if not mlp:
+            continue
+        out[p + "norm2"] = out[p + "norm2b"] = (W,)
+        f = p + "mlp."
+        if mlp["kind"] == "dense":
+            out[f + "gate"] = out[f + "up"] = (mlp["ff"], W)
+            out[f + "down"] = (W, mlp["ff"])
+        else:
+            ff = mlp["expert"]["ff"]
+            for k in range(mlp["router"]["experts"]):
+                out[f"{f}e{k}.gate"] = out[f"{f}e{k}.up"] = (ff, W)
+                out[f"{f}e{k}.down"] = (W, ff)
+            out[f + "router"] = (mlp["router"]["experts"], W)
+            if mlp.get("shared"):
+                sf = mlp["shared"]["ff"]
+                out[f + "shared.gate"] = out[f + "shared.up"] = (sf, W)
+                out[f + "shared.down"], out[f + "shared.sg"] = (W, sf), (1, W)
+    return out
+
+
+def sinulorn_pack(c: LayeredConfig, t: dict) -> dict:
+    """Checkpoint tensors (name -> array, bf16 bits as uint16 or floats, checkpoint shapes)
+    -> the engine's tensors: {"embed", "final_norm", "head", "layers": [field -> array]}."""
+    dt = c.weight_dtype
+
+    def w(*names):
+        parts = [_as_weight(t[n], dt) for n in names]
+        return parts[0] if len(parts) == 1 else np.ascontiguousarray(np.concatenate(parts, axis=0))
+
+    def f(*names):
+        parts = [_as_f32(t[n]).reshape(-1) if len(names) > 1 else _as_f32(t[n]) for n in names]
+        return np.ascontiguousarray(parts[0] if len(parts) == 1 else np.concatenate(parts))
+
+    layers = []
+    for i, l in enumerate(c.layers):
+        p, x, m = f"l{i}.", f"l{i}.mix.", f"l{i}.mlp."
+        d = {"norm1": f(p + "norm1"), "norm1b": f(p + "norm1b")}
+        if l.ff_kind != FF_NONE:
+            d.update(norm2=f(p + "norm2"), norm2b=f(p + "norm2b"))
+        if l.mixer == MIX_LATENT:
+            d["w_in"] = w(x + "dq", x + "dkv") if l.kv_from < 0 else w(x + "dq")
+            d["q_norm"] = f(x + "dq.norm")
+            if l.kv_from < 0:
+                d["kv_norm"] = f(x + "dkv.norm")
+            d["w_uq"] = w(x + "uq")
+            uk = _as_weight(t[x + "uk"], dt).reshape(l.heads, l.dim, l.kv_rank)
+            d["w_ukt"] = np.ascontiguousarray(uk.transpose(0, 2, 1))
+            d["w_uv"] = w(x + "uv")
+        elif l.mixer == MIX_RGLRU:
+            d["w_in"] = w(x + "y", x + "x")
+            d["in_bias"] = f(x + "y.b", x + "x.b")
+            d.update(conv_w=f(x + "conv"), conv_b=f(x + "conv.b"), gate_a=f(x + "ra"), gate_a_b=f(x + "ra.b").reshape(-1),
+                     gate_i=f(x + "ri"), gate_i_b=f(x + "ri.b").reshape(-1), lam=f(x + "lam"))
+        else:
+            d["w_in"] = w(x + "q", x + "k", x + "v", x + "g", x + "b", x + "a")
+            d["conv_w"] = np.ascontiguousarray(
+                np.concatenate([_as_f32(t[x + n + ".conv"]) for n in ("q", "k", "v")], axis=0))
+            d.update(a_log=f(x + "A_log"), dt_bias=f(x + "dt_bias"), out_norm=f(x + "norm"))
+        d["w_o"] = w(x + "o")
+        if l.ff_kind == FF_DENSE:
+            d.update(w_gate=w(m + "gate"), w_up=w(m + "up"), w_down=w(m + "down"))
+        elif l.ff_kind == FF_MOE:
+            d["router"] = f(m + "router")
+            for k in ("gate", "up", "down"):
+                d["w_" + k] = np.ascontiguousarray(
+                    np.stack([_as_weight(t[f"{m}e{e}.{k}"], dt) for e in range(l.experts)]))
+            if l.shared_ff:
+                d.update(shared_sg=f(m + "shared.sg").reshape(-1), ws_gate=w(m + "shared.gate"),
+                         ws_up=w(m + "shared.up"), ws_down=w(m + "shared.down"))
+        want = packed_shapes(c, l)
+        for k, (shape, _) in want.items():
+            if tuple(d[k].shape) != tuple(shape):
+                raise ValueError(f"layer {i}: tensor {k} has shape {d[k].shape}, the configuration gives {shape}")
+        layers.append(d)
+    return {"embed": w("embed"), "final_norm": f("final.norm"), "head": w("head"), "layers": layers}
+
+
+def sinulorn_random_tensors(cfg: dict, seed: int = 0, gain: float = 1.0) -> dict:
+    """Random checkpoint tensors for a Sinulorn config.json, as float32 arrays already
+    rounded to bf16 values (so the f32 and bf16 engines and a float64 restatement see the
+    same weights). Scales keep activations of order one through deep stacks."""
+    rng = np.random.default_rng(seed)
+    out = {}
+    for name, shape in sinulorn_tensor_shapes(cfg).items():
+        leaf = name.split(".")[-1]
+        if leaf in ("norm1", "norm2", "norm1b", "norm2b") or name.endswith((".norm", "final.norm")):
+            a = 1.0 + 0.2 * rng.standard_normal(shape)
+        elif leaf == "b" and len(shape) == 1 or name.endswith((".y.b", ".x.b", "conv.b", "ra.b", "ri.b")):
+            a = 0.3 * rng.standard_normal(shape)
+        elif leaf == "conv":
+            a = 0.5 * rng.standard_normal(shape)
+        elif leaf == "lam":
+            a = rng.uniform(-4.0, 1.0, shape)
+        elif leaf == "A_log":
+            a = rng.uniform(-3.0, 0.5, shape)
+        elif leaf == "dt_bias":
+            a = rng.uniform(-2.0, 1.0, shape)
+        elif leaf == "embed":
+            a = 0.1 * rng.standard_normal(shape)
+        else:
+            a = gain * rng.standard_normal(shape) / np.sqrt(shape[-1])
+        out[name] = bf16_to_f32(f32_to_bf16(a.astype(np.float32))).reshape(shape)
+    return out
+
+
+# ------------------------------------------------------------------ registry
+# design name (config.json "architecture") -> (config reader, weight packer)
+DESIGNS = {"Sinulorn": (sinulorn_config, sinulorn_pack)}
+
+
+def read_checkpoint(path: str, max_tokens: int = 4096, weight_dtype: int = M.BF16):
+    """A checkpoint folder -> (LayeredConfig, packed engine tensors). The design is
+    chosen by config.json's "architecture"."""
+    from .yalmfile import read_yalm
+
+    with open(os.path.join(path, "config.json")) as fh:
+        cfg = json.load(fh)
+    arch = cfg.get("architecture")
+    if arch not in DESIGNS:
+        raise ValueError(f"architecture {arch!r} is not a layer-list design this engine knows ({sorted(DESIGNS)})")
+    reader, packer = DESIGNS[arch]
+    c = reader(cfg, max_tokens, weight_dtype)
+    yd = read_yalm(os.path.join(path, "model.safetensors"))
+    try:
+        t = {k: np.asarray(v.data).reshape(v.shape) for k, v in yd.tensors.items()}
+        return c, packer(c, t)
+    finally:
+        yd.close()

@@ -19,6 +19,11 @@ from . import models as M
 HERE = os.path.dirname(os.path.abspath(__file__))
 # YALM_LIB: another build of the same ABI (A/B timing of two revisions, tools/build_ab_lib.sh)
 LIB_PATH = os.environ.get("YALM_LIB") or os.path.join(HERE, "libyalm_hip.so")
+# libyalm_seq.so: the device shim and the layer-list engine alone (`make seq`), for a tool
+# that serves only layer-list models; bound when the whole library has not been built
+PARTIAL = False
+if not os.path.exists(LIB_PATH) and not os.environ.get("YALM_LIB") and os.path.exists(os.path.join(HERE, "libyalm_seq.so")):
+    LIB_PATH, PARTIAL = os.path.join(HERE, "libyalm_seq.so"), True
 
 if not os.path.exists(LIB_PATH):
     raise ImportError(
@@ -73,8 +78,8 @@ class ModelWeights(ctypes.Structure):
 
 
 def _sig(name, restype, argtypes):
-    if os.environ.get("YALM_LIB") and not hasattr(lib, name):
-        return None  # an older build under A/B timing may lack newer entry points
+    if (os.environ.get("YALM_LIB") or PARTIAL) and not hasattr(lib, name):
+        return None  # an older build under A/B timing, or the layer-list library alone
     f = getattr(lib, name)
     f.restype = restype
     f.argtypes = argtypes
@@ -131,6 +136,48 @@ _sig("yalm_attn_prefill", c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int,
 _sig("yalm_set_prefill_forms", c_int, [c_void_p, ctypes.c_char_p])
 _sig("yalm_graph_kernels", c_int, [c_void_p, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int)])
 _sig("yalm_attn_wo_plan", c_int, [c_void_p, c_int, ctypes.POINTER(c_int), ctypes.POINTER(c_int)])
+
+# layer-list models (include/yalm_hip.h "layer-list models")
+class SeqLayer(ctypes.Structure):
+    """yalm_seq_layer."""
+
+    INTS = ("mixer", "heads", "kv_heads", "dim", "vdim", "kv_rank", "q_rank", "kv_from")
+    PTRS = ("norm1", "norm1b", "norm2", "norm2b", "q_norm", "kv_norm", "in_bias", "conv_w", "conv_b", "gate_a",
+            "gate_a_b", "gate_i", "gate_i_b", "lam", "a_log", "dt_bias", "out_norm", "router", "shared_sg",
+            "w_in", "w_uq", "w_ukt", "w_uv", "w_o", "w_gate", "w_up", "w_down", "ws_gate", "ws_up", "ws_down")
+    _fields_ = (
+        [(n, c_int) for n in INTS] + [("attn_scale", c_float), ("rec_width", c_int), ("blocks", c_int), ("conv", c_int),
+                                      ("ff_kind", c_int), ("ff", c_int), ("experts", c_int), ("top", c_int),
+                                      ("groups", c_int), ("groups_keep", c_int), ("router_scale", c_float),
+                                      ("limit", c_float), ("shared_ff", c_int), ("shared_limit", c_float)]
+        + [(n, c_void_p) for n in PTRS]
+    )
+
+
+class SeqConfig(ctypes.Structure):
+    _fields_ = [("width", c_int), ("vocab", c_int), ("n_layers", c_int), ("max_tokens", c_int),
+                ("embed_scale", c_float), ("norm_eps", c_float), ("weight_dtype", c_int)]
+
+
+class SeqWeights(ctypes.Structure):
+    _fields_ = [("embed", c_void_p), ("final_norm", c_void_p), ("head", c_void_p), ("layers", ctypes.POINTER(SeqLayer))]
+
+
+_sig("yalm_seq_create", c_int, [ctypes.POINTER(SeqConfig), ctypes.POINTER(SeqWeights), c_void_p,
+                                 ctypes.POINTER(c_void_p)])
+_sig("yalm_seq_destroy", c_int, [c_void_p])
+_sig("yalm_seq_reset", c_int, [c_void_p])
+_sig("yalm_seq_pos", c_int, [c_void_p, ctypes.POINTER(c_int)])
+_sig("yalm_seq_step", c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p])
+_sig("yalm_seq_generate_greedy", c_int, [c_void_p, c_int, c_int, c_void_p])
+_sig("yalm_seq_layer_dump", c_int, [c_void_p, c_int])
+_sig("yalm_seq_get_layers", c_int, [c_void_p, c_void_p, c_size_t])
+_sig("yalm_seq_time_step", c_int, [c_void_p, c_int, c_int, c_int, ctypes.POINTER(c_float)])
+
+SEQ_EXPORTED = [
+    "yalm_seq_create", "yalm_seq_destroy", "yalm_seq_reset", "yalm_seq_pos", "yalm_seq_step",
+    "yalm_seq_generate_greedy", "yalm_seq_layer_dump", "yalm_seq_get_layers", "yalm_seq_time_step",
+]
 
 EXPORTED = [
     "yalm_last_error", "yalm_set_device", "yalm_upload", "yalm_alloc", "yalm_download", "yalm_register_host",
@@ -580,3 +627,173 @@ class Decoder:
             self.close()
         except Exception:
             pass
+
+
+# ------------------------------------------------------------- layer-list models
+class SeqModel:
+    """A layer-list model's weights resident in HBM (layered.LayeredConfig + the packed
+    per-layer tensors of layered.packed_shapes)."""
+
+    def __init__(self, cfg):
+        self.cfg = cfg
+        self.ptrs: dict = {}
+        self.layer_ptrs: list = []
+        self._owned: list = []
+
+    def _up(self, a: np.ndarray) -> int:
+        a = np.ascontiguousarray(a)
+        p = lib.yalm_upload(a.ctypes.data, a.nbytes)
+        if not p:
+            raise YalmError(lib.yalm_last_error().decode())
+        self._owned.append(p)
+        return p
+
+    @classmethod
+    def from_packed(cls, cfg, packed: dict) -> "SeqModel":
+        self = cls(cfg)
+        for k in ("embed", "final_norm", "head"):
+            self.ptrs[k] = self._up(packed[k])
+        for d in packed["layers"]:
+            self.layer_ptrs.append({k: self._up(a) for k, a in d.items()})
+        return self
+
+    @classmethod
+    def from_checkpoint(cls, path: str, max_tokens: int = 4096, weight_dtype: int = M.BF16) -> "SeqModel":
+        from . import layered
+
+        cfg, packed = layered.read_checkpoint(path, max_tokens, weight_dtype)
+        return cls.from_packed(cfg, packed)
+
+    @classmethod
+    def synthetic(cls, cfg, seed: int = 1) -> "SeqModel":
+        """Random weights of cfg's shapes generated in HBM (yalm_synth): matrices uniform
+        with the usual 1 / sqrt(fan-in) spread, norms near 1, small biases and decays."""
+        from . import layered
+
+        self = cls(cfg)
+        wdt = cfg.weight_dtype
+
+        def make(name, shape, kind, fan_in=None):
+            n = int(np.prod(shape))
+            dt = wdt if kind == "w" else M.F32
+            nb = n * (2 if dt == M.BF16 else 4)
+            p = lib.yalm_alloc(nb)
+            if not p:
+                raise YalmError(lib.yalm_last_error().decode())
+            self._owned.append(p)
+            leaf = name.rsplit(".", 1)[-1]
+            if kind == "w" or leaf in ("router", "gate_a", "gate_i", "shared_sg"):
+                scale, off = 1.7 / np.sqrt(fan_in or shape[-1]), 0.0
+            elif leaf.startswith("norm") or leaf in ("q_norm", "kv_norm", "out_norm", "final_norm"):
+                scale, off = 0.2, 1.0
+            elif leaf == "conv_w":
+                scale, off = 0.5, 0.0
+            elif leaf in ("lam", "a_log", "dt_bias"):
+                scale, off = 1.5, -1.0
+            else:
+                scale, off = 0.3, 0.0
+            check(lib.yalm_synth(p, n, dt, M.synth_seed(seed, name), scale, off, None))
+            return p
+
+        self.ptrs["embed"] = make("embed", (cfg.vocab, cfg.width), "w", fan_in=100.0)
+        self.ptrs["final_norm"] = make("final_norm", (cfg.width,), "f")
+        self.ptrs["head"] = make("head", (cfg.vocab, cfg.width), "w")
+        for i, l in enumerate(cfg.layers):
+            self.layer_ptrs.append({k: make(f"l{i}.{k}", shape, kind)
+                                    for k, (shape, kind) in layered.packed_shapes(cfg, l).items()})
+        check(lib.yalm_stream_sync(None))
+        return self
+
+    def structs(self):
+        cfg = self.cfg
+        arr = (SeqLayer * len(cfg.layers))()
+        for i, (l, ptrs) in enumerate(zip(cfg.layers, self.layer_ptrs)):
+            for name, _ in SeqLayer._fields_:
+                if name in SeqLayer.PTRS:
+                    setattr(arr[i], name, ptrs.get(name))
+                else:
+                    setattr(arr[i], name, getattr(l, name))
+        sc = SeqConfig(cfg.width, cfg.vocab, len(cfg.layers), cfg.max_tokens, cfg.embed_scale, cfg.norm_eps,
+                       cfg.weight_dtype)
+        sw = SeqWeights(self.ptrs["embed"], self.ptrs["final_norm"], self.ptrs["head"], arr)
+        return sc, sw, arr
+
+    def close(self):
+        for p in self._owned:
+            lib.yalm_free(p)
+        self._owned = []
+        self.ptrs = {}
+        self.layer_ptrs = []
+
+
+class SeqDecoder:
+    """One sequence of a layer-list model on the device: latent caches, recurrent and
+    convolution states, position. step() appends tokens (a prompt, a portion of one, or a
+    single token); reset() ends the sequence and frees its states for the next one."""
+
+    def __init__(self, model: SeqModel):
+        self.model = model
+        self.cfg = model.cfg
+        self._sc, self._sw, self._arr = model.structs()
+        h = c_void_p()
+        check(lib.yalm_seq_create(ctypes.byref(self._sc), ctypes.byref(self._sw), None, ctypes.byref(h)))
+        self.h = h
+
+    @property
+    def pos(self) -> int:
+        p = c_int()
+        check(lib.yalm_seq_pos(self.h, ctypes.byref(p)))
+        return p.value
+
+    def reset(self) -> None:
+        check(lib.yalm_seq_reset(self.h))
+
+    def step(self, tokens, want=()):
+        """Append tokens; returns the logits [len(want), vocab] at the asked indices
+        (ascending, into tokens), or None."""
+        tok = np.ascontiguousarray(tokens, dtype=np.int32)
+        w = np.ascontiguousarray(want, dtype=np.int32)
+        out = np.empty((len(w), self.cfg.vocab), np.float32) if len(w) else None
+        check(lib.yalm_seq_step(self.h, _ptr(tok), len(tok), _ptr(w) if len(w) else None, len(w),
+                                _ptr(out) if len(w) else None))
+        return out
+
+    def generate_greedy(self, token: int, n: int) -> list:
+        out = np.zeros(max(n, 1), np.int32)
+        check(lib.yalm_seq_generate_greedy(self.h, token, n, out.ctypes.data))
+        return out[:n].tolist()
+
+    def layer_dump(self, on: bool = True) -> None:
+        check(lib.yalm_seq_layer_dump(self.h, int(on)))
+
+    def get_layers(self, n_tokens: int) -> np.ndarray:
+        out = np.empty((len(self.cfg.layers), n_tokens, self.cfg.width), np.float32)
+        check(lib.yalm_seq_get_layers(self.h, _ptr(out), out.size))
+        return out
+
+    def time_step(self, n: int, pos0: int = 0, iters: int = 3) -> float:
+        ms = c_float()
+        check(lib.yalm_seq_time_step(self.h, n, pos0, iters, ctypes.byref(ms)))
+        return ms.value
+
+    def close(self):
+        if getattr(self, "h", None):
+            check(lib.yalm_seq_destroy(self.h))
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def load_model(path: str, max_tokens: int = 4096, weight_dtype: int = None):
+    """A model folder or file -> (device model, decoder), the class chosen as the
+    framework does: a .yalm file is a Llama / Mistral decoder (DeviceModel + Decoder), a
+    folder whose config.json names a layer-list design is a SeqModel + SeqDecoder."""
+    if os.path.isdir(path):
+        m = SeqModel.from_checkpoint(path, max_tokens, M.BF16 if weight_dtype is None else weight_dtype)
+        return m, SeqDecoder(m)
+    m = DeviceModel.from_yalm(path, max_tokens)
+    return m, Decoder(m)
