@@ -74,6 +74,11 @@ def parse():
                     help="N > 1 on ONE GPU: every rank on device 0, its decoder stream on a disjoint block of "
                          "256/N CUs (yalm_stream_create_cu_part), IPC transport -- config 5's production launch "
                          "sequence rehearsed, not a scaling measurement")
+    ap.add_argument("--layered", action="store_true",
+                    help="instead of the default workload: prefill and decode throughput of the layer-list engine "
+                         "(Sinulorn-shaped stacks, random bf16 weights) at a few real layer sizes, each beside a "
+                         "Llama-shaped decoder of equal width, depth and feed-forward size; one JSON line")
+    ap.add_argument("--layered-sizes", default="1024,2048,4096", help="model widths of the --layered legs")
     return ap.parse_args()
 
 
@@ -504,8 +509,90 @@ def fp8_leg(args):
         return {"error": repr(e)[:300]}
 
 
+def layered_stack(Ly, M, width, max_tokens):
+    """A Sinulorn-shaped stack at a real layer size: every mixer and both feed-forward kinds,
+    head size 128, latent ranks in the usual proportions, experts whose active hidden size
+    (top x expert + shared) equals the dense layers' 3.5 x width."""
+    heads = width // 128
+    ff = width * 7 // 2
+    dense = dict(ff_kind=Ly.FF_DENSE, ff=ff)
+    moe = dict(ff_kind=Ly.FF_MOE, ff=ff // 8, experts=16, top=4, groups=4, groups_keep=2, router_scale=2.5, limit=7.0,
+               shared_ff=ff // 2, shared_limit=7.0)
+    lat = dict(heads=heads, dim=128, vdim=128, kv_rank=256, q_rank=max(width // 2, 256), attn_scale=128 ** -0.5)
+    layers = [
+        Ly.LayerSpec(Ly.MIX_DELTA, heads=heads, kv_heads=max(heads // 2, 1), dim=128, vdim=128, conv=4, **dense),
+        Ly.LayerSpec(Ly.MIX_LATENT, **lat, **moe),
+        Ly.LayerSpec(Ly.MIX_RGLRU, rec_width=width, blocks=heads, conv=4, **dense),
+        Ly.LayerSpec(Ly.MIX_DELTA, heads=heads, kv_heads=max(heads // 2, 1), dim=128, vdim=128, conv=4, **moe),
+        Ly.LayerSpec(Ly.MIX_LATENT, kv_from=1, **lat, **dense),
+        Ly.LayerSpec(Ly.MIX_RGLRU, rec_width=width, blocks=heads, conv=4, **dense),
+    ]
+    return Ly.LayeredConfig("Sinulorn", width, 32000, layers, embed_scale=1.0, norm_eps=1e-5, max_tokens=max_tokens,
+                            weight_dtype=M.BF16)
+
+
+def layered_bench(args, out_file):
+    """--layered: tokens/s of a prompt portion (n = 2048 at position 0) and of single-token
+    decoding (the device greedy loop at context ~1024) for the layer-list engine, and for a
+    Llama-shaped decoder (f16, the framework's MFMA prefill and fused decode) of the same
+    width, depth, feed-forward size and vocabulary. Random weights, synthetic ids."""
+    from yalm_amd import layered as Ly
+    from yalm_amd import models as M
+    from yalm_amd import runtime
+
+    runtime.check(runtime.lib.yalm_set_device(0))
+    n_pf, ctx, steps = 2048, 1024, max(args.steps if args.steps != 256 else 64, 8)
+    legs = []
+    for width in [int(x) for x in args.layered_sizes.split(",")]:
+        cfg = layered_stack(Ly, M, width, n_pf + 64)
+        model = runtime.SeqModel.synthetic(cfg, seed=3)
+        dec = runtime.SeqDecoder(model)
+        pf_ms = dec.time_step(n_pf, 0, max(args.prefill_iters, 1))
+        dec.reset()
+        dec.step([(7 * i + 1) % cfg.vocab for i in range(ctx)])
+        tok = dec.generate_greedy(1, args.warmup or 1)[-1]
+        t0 = time.perf_counter()
+        dec.generate_greedy(tok, steps)
+        dt = time.perf_counter() - t0
+        leg = {"width": width, "layers": len(cfg.layers), "prefill_tokens": n_pf, "prefill_ms": round(pf_ms, 3),
+               "prefill_tok_s": round(n_pf / pf_ms * 1e3, 1), "decode_context": ctx, "decode_steps": steps,
+               "decode_ms_per_token": round(dt / steps * 1e3, 4), "decode_tok_s": round(steps / dt, 2)}
+        dec.close()
+        model.close()
+        ref = M.ModelConfig(dim=width, hidden_dim=width * 7 // 2, head_dim=128, n_layers=len(cfg.layers),
+                            n_heads=width // 128, n_kv_heads=max(width // 512, 1), vocab_size=32000,
+                            max_seq_len=n_pf + 64, weight_dtype=M.F16)
+        dm = runtime.DeviceModel.synthetic(ref, seed=3)
+        rd = runtime.Decoder(dm)
+        try:
+            rpf = rd.prefill_time(n_pf, max(args.prefill_iters, 1))
+            rd.prefill([(7 * i + 1) % ref.vocab_size for i in range(ctx)], 0, logprobs=False)
+            rd.generate_greedy(1, ctx, args.warmup or 1)
+            t0 = time.perf_counter()
+            rd.enqueue_greedy(steps)
+            rd.device_step()
+            rdt = time.perf_counter() - t0
+            leg.update(ref_prefill_ms=round(rpf, 3), ref_prefill_tok_s=round(n_pf / rpf * 1e3, 1),
+                       ref_decode_ms_per_token=round(rdt / steps * 1e3, 4), ref_decode_tok_s=round(steps / rdt, 2))
+        except runtime.YalmError as e:
+            leg["ref_error"] = str(e)[:200]
+        finally:
+            rd.close()
+            dm.close()
+        legs.append(leg)
+    print(json.dumps({"metric": "layer-list engine (Sinulorn-shaped stack, bf16) prefill and decode tok/s beside a "
+                                "Llama-shaped f16 decoder of equal width / depth / feed-forward size @1 GPU",
+                      "n_gpus": 1, "dtype": "bf16", "data": "synthetic", "legs": legs}), file=out_file, flush=True)
+
+
 def main():
     args = parse()
+    if args.layered:
+        sys.stdout.flush()
+        real = os.fdopen(os.dup(1), "w")
+        os.dup2(2, 1)
+        layered_bench(args, real)
+        return
     if args.long_only:
         args.no_fp8 = args.no_gpu_state = True
     if "WORLD_SIZE" not in os.environ and args.gpus > 1:

@@ -68,24 +68,32 @@ def latent(cfg, w, pre, h, m, eps):
     return rms_norm(h @ w[pre + "dkv"].T, w[pre + "dkv.norm"], eps)
 
 
-def latent_attention(cfg, w, pre, h, m, eps, c):
-    """Causal softmax attention whose keys and values are up-projections of the
-    latent c [T, kv_rank] (this layer's own or another layer's)."""
+def attention_weights(cfg, w, pre, h, m, eps, c):
+    """Softmax weights [heads, T, T] of a latent-attention layer (row t over keys j <= t)."""
     T = h.shape[0]
-    H, D, V = m["heads"], m["dim"], m["vdim"]
+    H, D = m["heads"], m["dim"]
     cq = rms_norm(h @ w[pre + "dq"].T, w[pre + "dq.norm"], eps)
     q = (cq @ w[pre + "uq"].T).reshape(T, H, D)
     k = (c @ w[pre + "uk"].T).reshape(T, H, D)
-    v = (c @ w[pre + "uv"].T).reshape(T, H, V)
-    out = np.zeros((T, H, V), F)
     mask = np.tril(np.ones((T, T), bool))
+    P = np.zeros((H, T, T), F)
     for hh in range(H):
         s = (q[:, hh] @ k[:, hh].T) * m["scale"]
         s = np.where(mask, s, -np.inf)
         s = s - s.max(axis=1, keepdims=True)
         p = np.exp(s)
-        p /= p.sum(axis=1, keepdims=True)
-        out[:, hh] = p @ v[:, hh]
+        P[hh] = p / p.sum(axis=1, keepdims=True)
+    return P
+
+
+def latent_attention(cfg, w, pre, h, m, eps, c):
+    """Causal softmax attention whose keys and values are up-projections of the
+    latent c [T, kv_rank] (this layer's own or another layer's)."""
+    T = h.shape[0]
+    H, V = m["heads"], m["vdim"]
+    P = attention_weights(cfg, w, pre, h, m, eps, c)
+    v = (c @ w[pre + "uv"].T).reshape(T, H, V)
+    out = np.stack([P[hh] @ v[:, hh] for hh in range(H)], axis=1)
     return out.reshape(T, H * V) @ w[pre + "o"].T
 
 

@@ -78,8 +78,7 @@ static int in_rows(const yalm_seq_layer &l) {
 }
 
 static int validate(const yalm_seq_config &c, const std::vector<yalm_seq_layer> &L) {
-	ARGCHK(c.width > 0 && c.width % 2 == 0 && c.vocab > 0 && c.n_layers > 0 && c.max_tokens > 0,
-	       "yalm_seq_create: bad model sizes (width must be even)");
+	ARGCHK(c.width > 0 && c.vocab > 0 && c.n_layers > 0 && c.max_tokens > 0, "yalm_seq_create: bad model sizes");
 	ARGCHK(c.weight_dtype == YALM_BF16 || c.weight_dtype == YALM_F32, "yalm_seq_create: weight_dtype must be bf16 or f32");
 	for (int i = 0; i < c.n_layers; ++i) {
 		const yalm_seq_layer &l = L[i];
@@ -237,8 +236,8 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 	STRY(sallocT(q, &q->gen_tokens, q->gen_cap));
 	// position frequencies 10000^(-2 i / width), evaluated in double
 	{
-		std::vector<float> f(c.width / 2);
-		for (int i = 0; i < c.width / 2; ++i)
+		std::vector<float> f((c.width + 1) / 2);
+		for (int i = 0; i < (c.width + 1) / 2; ++i)
 			f[i] = (float)std::pow(10000.0, -2.0 * i / (double)c.width);
 		STRY(sallocT(q, &q->inv_freq, f.size()));
 		if (hipMemcpy(q->inv_freq, f.data(), f.size() * sizeof(float), hipMemcpyHostToDevice) != hipSuccess) {
@@ -321,6 +320,12 @@ static int gemm_t(Seq *q, const GemmArgs &a, int batches, int max_m) {
 			seq_gemv_kernel<WT, true><<<g, SEQ_THREADS, 0, q->stream>>>(a);
 		else
 			seq_gemv_kernel<WT, false><<<g, SEQ_THREADS, 0, q->stream>>>(a);
+	} else if (WT::BYTES == 2 && max_m > GT_BM) {
+		const dim3 g(cdiv(a.N, GB_BN), cdiv(max_m, GB_BM), batches);
+		if (glu)
+			seq_gemm_bf16_kernel<true><<<g, SEQ_THREADS, 0, q->stream>>>(a);
+		else
+			seq_gemm_bf16_kernel<false><<<g, SEQ_THREADS, 0, q->stream>>>(a);
 	} else {
 		const dim3 g(cdiv(a.N, GT_BN), cdiv(max_m, GT_BM), batches);
 		if (glu)

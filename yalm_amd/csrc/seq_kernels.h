@@ -457,6 +457,153 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_gemm_kernel(GemmArgs a) {
 	}
 }
 
+// ---- long portions, bf16: 128 x 128 output tiles, 4 waves of 64 x 64 (2 x 2 MFMA tiles of
+// 32 x 32), K in slabs of 32 through two LDS buffers: the next slab's global loads (and the
+// activations' f32 -> bf16 rounding) are issued before the current slab's 8 MFMAs per wave
+// and stored to the other buffer after them, one barrier per slab.
+#define GB_BM 128
+#define GB_BN 128
+template <bool GLU>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_gemm_bf16_kernel(GemmArgs a) {
+	const GemmBatch b = gemm_batch<WBF16>(a, blockIdx.z);
+	const int m0 = blockIdx.y * GB_BM, n0 = blockIdx.x * GB_BN;
+	if (m0 >= b.M)
+		return;
+	constexpr int LD = GT_BK + 8;
+	__shared__ int arow[GB_BM], crow[GB_BM];
+	__shared__ __attribute__((aligned(16))) uint16_t As[2][GB_BM * LD], Bs[2][GB_BN * LD],
+	    Bs2[GLU ? 2 : 1][GLU ? GB_BN * LD : 8];
+	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+	if (tid < GB_BM) {
+		const int m = m0 + tid;
+		int ra = -1, rc = -1;
+		if (m < b.M) {
+			const int s = b.rows ? b.rows[m] : m;
+			ra = b.rows ? s / a.a_div : s;
+			rc = (b.rows && !a.c_dense) ? s : m;
+		}
+		arow[tid] = ra;
+		crow[tid] = rc;
+	}
+	__syncthreads();
+	const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;
+	const int lr = tid >> 2, lk = (tid & 3) * 8; // loader: rows lr and lr + 64, first k of 8
+	const int ra0 = arow[lr], ra1 = arow[lr + 64];
+	const bool avec = a.lda % 4 == 0 && (size_t)b.A % 16 == 0;
+	const bool wvec = a.ldw % 8 == 0 && ((size_t)b.W | (size_t)(GLU ? b.W2 : b.W)) % 16 == 0;
+	u32x4_t pa[2], pb[2], pb2[2];
+	auto fetch = [&](int k0) {
+		const int k = k0 + lk;
+#pragma unroll
+		for (int h = 0; h < 2; ++h) {
+			const int ra = h ? ra1 : ra0;
+			pa[h] = u32x4_t{0, 0, 0, 0};
+			if (ra >= 0) {
+				const float *src = b.A + (size_t)ra * a.lda + k;
+				float x[8];
+				if (avec && k + 8 <= a.K) {
+					const float4_t x0 = *(const float4_t *)src, x1 = *(const float4_t *)(src + 4);
+#pragma unroll
+					for (int e = 0; e < 4; ++e) {
+						x[e] = x0[e];
+						x[4 + e] = x1[e];
+					}
+				} else {
+#pragma unroll
+					for (int e = 0; e < 8; ++e)
+						x[e] = k + e < a.K ? src[e] : 0.0f;
+				}
+#pragma unroll
+				for (int e = 0; e < 4; ++e)
+					pa[h][e] = (uint32_t)f2bf(x[2 * e]) | ((uint32_t)f2bf(x[2 * e + 1]) << 16);
+			}
+			const int nb = n0 + lr + 64 * h;
+			pb[h] = u32x4_t{0, 0, 0, 0};
+			pb2[h] = u32x4_t{0, 0, 0, 0};
+			if (nb < a.N) {
+				const uint16_t *src = (const uint16_t *)b.W + (size_t)nb * a.ldw + k;
+				const uint16_t *src2 = GLU ? (const uint16_t *)b.W2 + (size_t)nb * a.ldw + k : nullptr;
+				if (wvec && k + 8 <= a.K) {
+					pb[h] = load16(src);
+					if constexpr (GLU)
+						pb2[h] = load16(src2);
+				} else {
+#pragma unroll
+					for (int e = 0; e < 4; ++e) {
+						const uint32_t lo = k + 2 * e < a.K ? src[2 * e] : 0, hi = k + 2 * e + 1 < a.K ? src[2 * e + 1] : 0;
+						pb[h][e] = lo | (hi << 16);
+						if constexpr (GLU) {
+							const uint32_t lo2 = k + 2 * e < a.K ? src2[2 * e] : 0,
+							               hi2 = k + 2 * e + 1 < a.K ? src2[2 * e + 1] : 0;
+							pb2[h][e] = lo2 | (hi2 << 16);
+						}
+					}
+				}
+			}
+		}
+	};
+	auto stash = [&](int buf) {
+#pragma unroll
+		for (int h = 0; h < 2; ++h) {
+			*(u32x4_t *)(As[buf] + (lr + 64 * h) * LD + lk) = pa[h];
+			*(u32x4_t *)(Bs[buf] + (lr + 64 * h) * LD + lk) = pb[h];
+			if constexpr (GLU)
+				*(u32x4_t *)(Bs2[buf] + (lr + 64 * h) * LD + lk) = pb2[h];
+		}
+	};
+	float16_t acc[2][2] = {}, acc2[GLU ? 2 : 1][GLU ? 2 : 1] = {};
+	fetch(0);
+	stash(0);
+	__syncthreads();
+	int buf = 0;
+	for (int k0 = 0; k0 < a.K; k0 += GT_BK) {
+		const bool more = k0 + GT_BK < a.K;
+		if (more)
+			fetch(k0 + GT_BK);
+#pragma unroll
+		for (int ks = 0; ks < GT_BK; ks += 16) {
+			const int kk = ks + 8 * (lane >> 5);
+			bf16x8_t fa[2], fb[2], fb2[2];
+#pragma unroll
+			for (int i = 0; i < 2; ++i) {
+				fa[i] = __builtin_bit_cast(bf16x8_t, *(const u32x4_t *)(As[buf] + (wm + 32 * i + (lane & 31)) * LD + kk));
+				fb[i] = __builtin_bit_cast(bf16x8_t, *(const u32x4_t *)(Bs[buf] + (wn + 32 * i + (lane & 31)) * LD + kk));
+				if constexpr (GLU)
+					fb2[i] = __builtin_bit_cast(bf16x8_t,
+					                            *(const u32x4_t *)(Bs2[buf] + (wn + 32 * i + (lane & 31)) * LD + kk));
+			}
+#pragma unroll
+			for (int i = 0; i < 2; ++i)
+#pragma unroll
+				for (int j = 0; j < 2; ++j) {
+					acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+					if constexpr (GLU)
+						acc2[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb2[j], acc2[i][j], 0, 0, 0);
+				}
+		}
+		if (more)
+			stash(buf ^ 1); // the other buffer: its last readers passed the previous barrier
+		__syncthreads();
+		buf ^= 1;
+	}
+#pragma unroll
+	for (int j = 0; j < 2; ++j) {
+		const int n = n0 + wn + 32 * j + (lane & 31);
+		if (n >= a.N)
+			continue;
+		const float bias = b.bias ? b.bias[n] : 0.0f;
+#pragma unroll
+		for (int i = 0; i < 2; ++i)
+#pragma unroll
+			for (int r = 0; r < 16; ++r) {
+				const int ml = wm + 32 * i + (r & 3) + 8 * (r >> 2) + 4 * (lane >> 5);
+				const int rc = crow[ml];
+				if (rc >= 0)
+					b.C[(size_t)rc * a.ldc + n] = epi_apply(a, acc[i][j][r], GLU ? acc2[i][j][r] : 0.0f, bias);
+			}
+	}
+}
+
 // ------------------------------------------------------------------ short causal convolution
 // out[t][c] = act(bias[c] + sum_j w[c][j] in(t - (taps - 1) + j)), in(tau) = Z[tau][col0 + c] for
 // tau >= 0, else the sequence's stored last inputs state[(taps - 1) + tau][c] (zeros at the start).

@@ -61,7 +61,14 @@ extern "C" int yalm_download(void *host, const void *device, size_t size) {
 }
 
 extern "C" int yalm_register_host(void *host, size_t size) {
-	HIPCHK(hipHostRegister(host, size, hipHostRegisterDefault));
+	// some hosts refuse to pin memory that already exists; the error must not stay behind
+	// for the next HIP call to report
+	const hipError_t e = hipHostRegister(host, size, hipHostRegisterDefault);
+	if (e != hipSuccess) {
+		(void)hipGetLastError();
+		set_err(std::string("hipHostRegister failed: ") + hipGetErrorString(e));
+		return YALM_ERR_HIP;
+	}
 	return YALM_OK;
 }
 

@@ -117,7 +117,7 @@ InferenceState::InferenceState(std::shared_ptr<Config> config) : _config(std::mo
 InferenceState::~InferenceState() {
 	if (_decoder)
 		yalm_decoder_destroy(_decoder);
-	if (_device == Device::HIP)
+	if (_pinned)
 		yalm_unregister_host(_logits);
 	delete[] _logits;
 }
@@ -126,8 +126,9 @@ void InferenceState::cuda() {
 	if (_device != Device::CPU)
 		return;
 	_device = Device::HIP;
-	// pinned logits so the OUTPUT copy is a straight DMA (model.cpp:338)
-	check(yalm_register_host(_logits, sizeof(float) * _config->vocab_size), "register logits");
+	// pinned logits so the OUTPUT copy is a straight DMA (model.cpp:338); where the host
+	// refuses to pin existing memory the copy goes through pageable memory instead
+	_pinned = yalm_register_host(_logits, sizeof(float) * _config->vocab_size) == YALM_OK;
 }
 
 Block::Block(int layer_i, std::shared_ptr<Config> config, const Tensor *rms_att_weight, const Tensor *rms_ffn_weight,

@@ -84,6 +84,7 @@ private:
 	Device _device = Device::CPU;
 	InferenceMode _mode = InferenceMode::OUTPUT_LOGITS;
 	float *_logits = nullptr;
+	bool _pinned = false; // _logits registered with the device
 	yalm_decoder _decoder = nullptr;
 };
 

@@ -191,6 +191,7 @@ EXPORTED = [
     "yalm_argmax", "yalm_set_prefill_forms", "yalm_attn_wo_plan", "yalm_graph_kernels",
     "yalm_stream_create_cu_part", "yalm_decoder_set_launch", "yalm_prefill_info", "yalm_set_prefill_precision",
 ]
+EXPORTED += SEQ_EXPORTED
 PREFILL_FAST, PREFILL_SPLIT = 0, 1  # yalm_set_prefill_precision
 
 HYDRATE_KV_CACHE, OUTPUT_LOGITS = 0, 1
