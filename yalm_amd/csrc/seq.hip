@@ -37,6 +37,8 @@ struct yalm_seq_s {
 	float *logits = nullptr;     // [LOGIT_ROWS][vocab]
 	int *idx = nullptr, *counts = nullptr, *lists = nullptr;
 	float *wt = nullptr, *sgate = nullptr;
+	float *att_part = nullptr;   // latent attention: per (row, key split) partial sums, maximum, sum
+	int att_splits = 1;          // key splits of single-token / short-portion attention
 	float *arena = nullptr;      // every recurrent and convolution state of the sequence
 	size_t arena_floats = 0;
 	std::vector<void *> cache;   // per layer: [max_tokens][kv_rank] latent rows (own latent only)
@@ -149,12 +151,10 @@ static int att_attr(int rank) {
 }
 template <class CT>
 static int att_attr_ct(int rank) {
-	const int na = cdiv(rank, 16);
+	const int na = cdiv(att_rank4(rank), 64);
 	if (na <= 1) return att_attr<CT, 1>(rank);
 	if (na <= 2) return att_attr<CT, 2>(rank);
-	if (na <= 4) return att_attr<CT, 4>(rank);
-	if (na <= 8) return att_attr<CT, 8>(rank);
-	return att_attr<CT, 16>(rank);
+	return att_attr<CT, 4>(rank);
 }
 
 static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, yalm_stream s, Seq **out) {
@@ -232,6 +232,16 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 	STRY(sallocT(q, &q->sgate, cap));
 	STRY(sallocT(q, &q->counts, max_e));
 	STRY(sallocT(q, &q->lists, (size_t)max_e * cap));
+	{
+		int max_h = 1, max_rank = 4;
+		for (const yalm_seq_layer &l : q->L)
+			if (l.mixer == YALM_MIX_LATENT) {
+				max_h = std::max(max_h, l.heads);
+				max_rank = std::max(max_rank, l.kv_rank);
+			}
+		q->att_splits = std::max(1, std::min(32, cdiv(c.max_tokens, 2 * ATT_KT)));
+		STRY(sallocT(q, &q->att_part, (size_t)(4 * ATT_BR + GEMV_MAX_M * max_h) * q->att_splits * (att_rank4(max_rank) + 4)));
+	}
 	q->gen_cap = 1 << 16;
 	STRY(sallocT(q, &q->gen_tokens, q->gen_cap));
 	// position frequencies 10000^(-2 i / width), evaluated in double
@@ -361,17 +371,20 @@ static GemmArgs plain(const float *A, int lda, const void *W, int ldw, float *C,
 template <class CT>
 static int attn_t(Seq *q, const float *Qa, const void *cache, int rank, int H, int n, float scale, float *ctx) {
 	const int NR = n * H;
-	const dim3 g(cdiv(NR, ATT_BR));
+	// few rows (single tokens, short portions): the visible keys are split over workgroups
+	const int S = NR <= 4 * ATT_BR ? q->att_splits : 1;
+	const dim3 g(cdiv(NR, ATT_BR), S);
 	const size_t lds = att_lds_bytes(rank);
-	const int na = cdiv(rank, 16);
+	const int na = cdiv(att_rank4(rank), 64);
 #define ATT_LAUNCH(NA)                                                                                                 \
-	seq_latent_attn_kernel<CT, NA><<<g, SEQ_THREADS, lds, q->stream>>>(Qa, (const CT *)cache, rank, H, NR, scale, q->st, ctx)
+	seq_latent_attn_kernel<CT, NA><<<g, SEQ_THREADS, lds, q->stream>>>(Qa, (const CT *)cache, rank, H, NR, scale, q->st, ctx, \
+	                                                                  q->att_part)
 	if (na <= 1) ATT_LAUNCH(1);
 	else if (na <= 2) ATT_LAUNCH(2);
-	else if (na <= 4) ATT_LAUNCH(4);
-	else if (na <= 8) ATT_LAUNCH(8);
-	else ATT_LAUNCH(16);
+	else ATT_LAUNCH(4);
 #undef ATT_LAUNCH
+	if (S > 1)
+		seq_latent_merge_kernel<<<NR, 64, 0, q->stream>>>(q->att_part, S, rank, ctx);
 	HIPCHK(hipGetLastError());
 	return YALM_OK;
 }
@@ -445,8 +458,14 @@ static int mixer_rglru(Seq *q, int li, int n) {
 		a.epi = EPI_SIGMOID;
 		TRY(gemm(q, a, l.blocks, -1, true));
 	}
-	seq_rglru_scan_kernel<<<cdiv(W, SEQ_THREADS), SEQ_THREADS, 0, q->stream>>>(r, ig, u, W, q->Z, 2 * W, l.lam, q->S[li],
-	                                                                           so, n);
+	if (n <= GEMV_MAX_M) {
+		seq_rglru_scan_kernel<<<cdiv(W, SEQ_THREADS), SEQ_THREADS, 0, q->stream>>>(r, ig, u, W, q->Z, 2 * W, l.lam,
+		                                                                           q->S[li], so, n);
+	} else {
+		seq_rglru_coef_kernel<<<dim3(cdiv(W, SEQ_THREADS), n), SEQ_THREADS, 0, q->stream>>>(r, ig, u, W, q->Z, 2 * W, l.lam,
+		                                                                                 n);
+		seq_rglru_walk_kernel<<<cdiv(W, SEQ_THREADS), SEQ_THREADS, 0, q->stream>>>(r, ig, u, W, q->S[li], so, n);
+	}
 	HIPCHK(hipGetLastError());
 	return gemm(q, plain(so, W, l.w_o, W, q->Y, c.width, n, c.width, W));
 }
@@ -490,7 +509,7 @@ static int ff_moe(Seq *q, int li, int n) {
 	const yalm_seq_config &c = q->c;
 	const int E = l.experts, top = l.top, ff = l.ff, slots = n * top;
 	float *hx = q->B[0], *yx = q->B[1], *hs = q->B[2], *ys = q->B[3];
-	seq_router_kernel<<<n, SEQ_THREADS, E * sizeof(float), q->stream>>>(q->Hn, c.width, l.router, E, top, l.groups,
+	seq_router_kernel<<<n, SEQ_THREADS, (E + l.groups) * sizeof(float), q->stream>>>(q->Hn, c.width, l.router, E, top, l.groups,
 	                                                                    l.groups_keep, l.router_scale,
 	                                                                    l.shared_ff > 0 ? l.shared_sg : nullptr, q->idx,
 	                                                                    q->wt, q->sgate);

@@ -674,6 +674,41 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_rglru_scan_kernel(const float
 	state[c] = S;
 }
 
+// Long portions: everything that does not depend on the carried state is evaluated for all
+// tokens at once (R <- a, I <- sqrt(1 - a^2) i u, U <- gelu_tanh(gate branch)), so that the
+// sequential walk below is one fused multiply-add per token and channel.
+__global__ __launch_bounds__(SEQ_THREADS) void seq_rglru_coef_kernel(float *__restrict__ R, float *__restrict__ I,
+                                                                     float *__restrict__ U, int W,
+                                                                     const float *__restrict__ Z, int ldz,
+                                                                     const float *__restrict__ lam, int T) {
+	const int c = blockIdx.x * SEQ_THREADS + threadIdx.x;
+	const int t = blockIdx.y;
+	if (c >= W)
+		return;
+	const size_t o = (size_t)t * W + c;
+	const float la = -8.0f * R[o] * sq_softplus(lam[c]);
+	R[o] = expf(la);
+	I[o] = sqrtf(-expm1f(2.0f * la)) * (I[o] * U[o]);
+	U[o] = sq_gelu_tanh(Z[(size_t)t * ldz + c]);
+}
+__global__ __launch_bounds__(SEQ_THREADS) void seq_rglru_walk_kernel(const float *__restrict__ A,
+                                                                     const float *__restrict__ B,
+                                                                     const float *__restrict__ G, int W,
+                                                                     float *__restrict__ state, float *__restrict__ out,
+                                                                     int T) {
+	const int c = blockIdx.x * SEQ_THREADS + threadIdx.x;
+	if (c >= W)
+		return;
+	float S = state[c];
+#pragma unroll 8
+	for (int t = 0; t < T; ++t) {
+		const size_t o = (size_t)t * W + c;
+		S = fmaf(A[o], S, B[o]);
+		out[o] = S * G[o];
+	}
+	state[c] = S;
+}
+
 // ------------------------------------------------------------------ gated delta rule
 // After the convolutions: q and k to unit length per head (q also x dim^-1/2), beta =
 // sigmoid, decay g = exp(-exp(a_log) softplus(a + dt_bias)). QKV: [T][ldq] = q | k | v
@@ -712,8 +747,8 @@ __device__ __forceinline__ float sum8(float v) { // over aligned groups of 8 lan
 }
 
 // The recurrence itself. The columns of a head's [dim][vdim] state never mix, so one group
-// of 8 lanes owns one column (its dim entries interleaved over the lanes, R per lane, in
-// registers) and walks the portion's tokens in order:
+// of 8 lanes owns one column (each lane a contiguous slice of R dim entries, in registers)
+// and walks the portion's tokens in order:
 //   S *= g;  u = beta (v - S.k);  S += k u;  o = S.q
 // (the read-out after the write). The next token's operands are loaded while the current
 // one is applied. grid (ceil(vdim / 32), heads).
@@ -726,22 +761,35 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__r
 	const int col = blockIdx.x * (SEQ_THREADS / 8) + (threadIdx.x >> 3), sub = threadIdx.x & 7;
 	const bool live = col < V;
 	const int vc = live ? col : V - 1;
+	const int d0 = sub * R; // this lane's slice of the key dimension: d0 .. d0 + R - 1
 	float S[R];
 	float *sp = state + (size_t)h * D * V;
 #pragma unroll
-	for (int i = 0; i < R; ++i) {
-		const int d = sub + 8 * i;
-		S[i] = (d < D) ? sp[(size_t)d * V + vc] : 0.0f;
-	}
+	for (int i = 0; i < R; ++i)
+		S[i] = (d0 + i < D) ? sp[(size_t)(d0 + i) * V + vc] : 0.0f;
 	const int qo = kh * D, ko = KH * D + kh * D, vo = 2 * KH * D + h * V + vc;
+	// 16-byte loads when every lane's slice is whole and aligned
+	const bool vec = R % 4 == 0 && D % R == 0 && ldq % 4 == 0 && qo % 4 == 0 && ko % 4 == 0 && (size_t)QKV % 16 == 0;
+	const bool inside = d0 + R <= D;
 	float kn[R], qn[R], vn, bn, gn;
 	auto load = [&](int t) {
 		const float *row = QKV + (size_t)t * ldq;
+		if (vec && inside) {
 #pragma unroll
-		for (int i = 0; i < R; ++i) {
-			const int d = sub + 8 * i;
-			kn[i] = d < D ? row[ko + d] : 0.0f;
-			qn[i] = d < D ? row[qo + d] : 0.0f;
+			for (int i = 0; i < R / 4; ++i) {
+				const float4_t k4 = *(const float4_t *)(row + ko + d0 + 4 * i), q4 = *(const float4_t *)(row + qo + d0 + 4 * i);
+#pragma unroll
+				for (int e = 0; e < 4; ++e) {
+					kn[4 * i + e] = k4[e];
+					qn[4 * i + e] = q4[e];
+				}
+			}
+		} else {
+#pragma unroll
+			for (int i = 0; i < R; ++i) {
+				kn[i] = d0 + i < D ? row[ko + d0 + i] : 0.0f;
+				qn[i] = d0 + i < D ? row[qo + d0 + i] : 0.0f;
+			}
 		}
 		vn = row[vo];
 		bn = BG[(size_t)t * 2 * H + h];
@@ -758,16 +806,16 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__r
 		const float v = vn, beta = bn, g = gn;
 		if (t + 1 < T)
 			load(t + 1);
-		float d0 = 0.0f, d1 = 0.0f;
+		float dd0 = 0.0f, dd1 = 0.0f;
 #pragma unroll
 		for (int i = 0; i < R; ++i) {
 			S[i] *= g;
 			if (i & 1)
-				d1 = fmaf(S[i], k[i], d1);
+				dd1 = fmaf(S[i], k[i], dd1);
 			else
-				d0 = fmaf(S[i], k[i], d0);
+				dd0 = fmaf(S[i], k[i], dd0);
 		}
-		const float u = beta * (v - sum8(d0 + d1));
+		const float u = beta * (v - sum8(dd0 + dd1));
 		float o0 = 0.0f, o1 = 0.0f;
 #pragma unroll
 		for (int i = 0; i < R; ++i) {
@@ -783,11 +831,9 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__r
 	}
 	if (live) {
 #pragma unroll
-		for (int i = 0; i < R; ++i) {
-			const int d = sub + 8 * i;
-			if (d < D)
-				sp[(size_t)d * V + col] = S[i];
-		}
+		for (int i = 0; i < R; ++i)
+			if (d0 + i < D)
+				sp[(size_t)(d0 + i) * V + col] = S[i];
 	}
 }
 
@@ -819,33 +865,52 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_out_kernel(const float 
 // multi-query attention with key = value = c. Rows r = t * H + h of Qa / Ctx; row r sees
 // cache rows j <= st->pos + r / H. Scores, softmax (running maximum and sum per row) and the
 // weighted sums are f32. A workgroup owns ATT_BR rows and walks the keys in tiles of 64:
-// each wave scores 4 rows x 64 keys (a lane per key), then every thread updates NACC
-// (row, latent entry) sums. Dynamic LDS: att_lds_bytes(rank).
+// each wave scores 4 rows x 64 keys (a lane per key), then every thread updates NA4 groups
+// of 4 latent entries of one row. Dynamic LDS: att_lds_bytes(rank).
 #define ATT_BR 16
 #define ATT_KT 64
-template <class CT, int NACC>
+// LDS rows are padded to a multiple of 4 floats (zeros) so that both phases read 16 bytes
+// at a time. Key splits (gridDim.y = S > 1, single tokens and short portions): split s walks
+// its share of the visible keys and leaves (sums, running maximum, running sum) per row in
+// `part` for seq_latent_merge_kernel; S == 1 writes the normalised sums to Ctx.
+__host__ __device__ inline int att_rank4(int rank) {
+	return (rank + 3) & ~3;
+}
+template <class CT, int NA4>
 __global__ __launch_bounds__(SEQ_THREADS) void seq_latent_attn_kernel(const float *__restrict__ Qa,
                                                                       const CT *__restrict__ cache, int rank, int H,
                                                                       int NR, float scale,
                                                                       const StepState *__restrict__ st,
-                                                                      float *__restrict__ Ctx) {
-	extern __shared__ float lds[];
-	const int ldc = rank + 1;
-	float *qs = lds;                      // [ATT_BR][rank]
-	float *cs = qs + ATT_BR * rank;       // [ATT_KT][rank + 1]
+                                                                      float *__restrict__ Ctx,
+                                                                      float *__restrict__ part) {
+	extern __shared__ __attribute__((aligned(16))) float lds[];
+	const int rank4 = att_rank4(rank), ldc = rank4 + 4, q4n = rank4 >> 2;
+	float *qs = lds;                      // [ATT_BR][rank4]
+	float *cs = qs + ATT_BR * rank4;      // [ATT_KT][rank4 + 4]
 	float *ps = cs + ATT_KT * ldc;        // [ATT_BR][ATT_KT]
 	float *alpha = ps + ATT_BR * ATT_KT;  // [ATT_BR]
 	float *lsum = alpha + ATT_BR;         // [ATT_BR]
+	float *mfin = lsum + ATT_BR;          // [ATT_BR]
 	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
 	const int r0 = blockIdx.x * ATT_BR;
+	const int S = gridDim.y, split = blockIdx.y;
 	const int pos0 = st->pos;
 	const int rlast = min(r0 + ATT_BR, NR) - 1;
-	const int kmax = pos0 + rlast / H; // the last visible key of the workgroup's last row
-	for (int i = tid; i < ATT_BR * rank; i += SEQ_THREADS) {
-		const int r = r0 + i / rank;
-		qs[i] = r < NR ? Qa[(size_t)r * rank + i % rank] * scale : 0.0f;
+	const int nkeys = pos0 + rlast / H + 1; // keys visible to the workgroup's last row
+	int k_begin = 0, k_end = nkeys;
+	if (S > 1) {
+		const int chunk = (((nkeys + S - 1) / S) + ATT_KT - 1) & ~(ATT_KT - 1);
+		k_begin = split * chunk;
+		k_end = min(nkeys, k_begin + chunk);
 	}
-	float acc[NACC] = {};
+	for (int i = tid; i < ATT_BR * rank4; i += SEQ_THREADS) {
+		const int r = r0 + i / rank4, d = i % rank4;
+		qs[i] = (r < NR && d < rank) ? Qa[(size_t)r * rank + d] * scale : 0.0f;
+	}
+	float4_t acc[NA4];
+#pragma unroll
+	for (int a = 0; a < NA4; ++a)
+		acc[a] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
 	float mrun[4], lrun[4];
 	int lim[4];
 #pragma unroll
@@ -853,31 +918,36 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_latent_attn_kernel(const floa
 		const int r = r0 + wave * 4 + i;
 		mrun[i] = -FLT_MAX;
 		lrun[i] = 0.0f;
-		lim[i] = r < NR ? pos0 + r / H : -1;
+		lim[i] = r < NR ? min(pos0 + r / H, k_end - 1) : -1;
 	}
-	for (int kt = 0; kt <= kmax; kt += ATT_KT) {
+	for (int kt = k_begin; kt < k_end; kt += ATT_KT) {
 		__syncthreads(); // the previous tile's sums have read cs / ps
-		for (int i = tid; i < ATT_KT * rank; i += SEQ_THREADS) {
-			const int j = kt + i / rank, d = i % rank;
+		for (int i = tid; i < ATT_KT * rank4; i += SEQ_THREADS) {
+			const int jj = i / rank4, d = i % rank4, j = kt + jj;
 			float v = 0.0f;
-			if (j <= kmax) {
+			if (j < k_end && d < rank) {
 				if constexpr (sizeof(CT) == 2)
 					v = bf2f(cache[(size_t)j * rank + d]);
 				else
 					v = cache[(size_t)j * rank + d];
 			}
-			cs[(i / rank) * ldc + d] = v;
+			cs[jj * ldc + d] = v;
 		}
 		__syncthreads();
 		{
 			float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-			const float *cj = cs + lane * ldc;
-			const float *q0 = qs + (wave * 4) * rank;
-			for (int d = 0; d < rank; ++d) {
-				const float c = cj[d];
+			const float4_t *cj = (const float4_t *)(cs + lane * ldc);
+			const float4_t *q0 = (const float4_t *)(qs + (wave * 4) * rank4);
+			for (int d = 0; d < q4n; ++d) {
+				const float4_t c = cj[d];
 #pragma unroll
-				for (int i = 0; i < 4; ++i)
-					s[i] = fmaf(q0[i * rank + d], c, s[i]);
+				for (int i = 0; i < 4; ++i) {
+					const float4_t qv = q0[i * q4n + d];
+					s[i] = fmaf(qv[0], c[0], s[i]);
+					s[i] = fmaf(qv[1], c[1], s[i]);
+					s[i] = fmaf(qv[2], c[2], s[i]);
+					s[i] = fmaf(qv[3], c[3], s[i]);
+				}
 			}
 #pragma unroll
 			for (int i = 0; i < 4; ++i) {
@@ -886,7 +956,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_latent_attn_kernel(const floa
 				const float mx = wave_max(sv);
 				const float mnew = fmaxf(mrun[i], mx);
 				const float p = vis ? expf(sv - mnew) : 0.0f;
-				const float al = expf(mrun[i] - mnew); // 1 when nothing is visible yet, 0 after the first key
+				const float al = expf(mrun[i] - mnew); // 1 while nothing is visible yet, 0 at the first key
 				lrun[i] = lrun[i] * al + wave_sum(p);
 				mrun[i] = mnew;
 				ps[(wave * 4 + i) * ATT_KT + lane] = p;
@@ -896,44 +966,94 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_latent_attn_kernel(const floa
 		}
 		__syncthreads();
 #pragma unroll
-		for (int a = 0; a < NACC; ++a) {
-			const int idx = tid + a * SEQ_THREADS;
-			if (idx < ATT_BR * rank) {
-				const int r = idx / rank, d = idx % rank;
-				float v = acc[a] * alpha[r];
-				const float *pr = ps + r * ATT_KT;
-#pragma unroll 8
-				for (int j = 0; j < ATT_KT; ++j)
-					v = fmaf(pr[j], cs[j * ldc + d], v);
+		for (int a = 0; a < NA4; ++a) {
+			const int u = tid + a * SEQ_THREADS;
+			if (u < ATT_BR * q4n) {
+				const int r = u / q4n, d4 = u % q4n;
+				const float al = alpha[r];
+				float4_t v = acc[a];
+				v[0] *= al;
+				v[1] *= al;
+				v[2] *= al;
+				v[3] *= al;
+				const float4_t *pr = (const float4_t *)(ps + r * ATT_KT);
+#pragma unroll 4
+				for (int j4 = 0; j4 < ATT_KT / 4; ++j4) {
+					const float4_t p = pr[j4];
+#pragma unroll
+					for (int e = 0; e < 4; ++e) {
+						const float4_t c = *(const float4_t *)(cs + (4 * j4 + e) * ldc + 4 * d4);
+						v[0] = fmaf(p[e], c[0], v[0]);
+						v[1] = fmaf(p[e], c[1], v[1]);
+						v[2] = fmaf(p[e], c[2], v[2]);
+						v[3] = fmaf(p[e], c[3], v[3]);
+					}
+				}
 				acc[a] = v;
 			}
 		}
 	}
 	if (lane == 0) {
 #pragma unroll
-		for (int i = 0; i < 4; ++i)
+		for (int i = 0; i < 4; ++i) {
 			lsum[wave * 4 + i] = lrun[i];
+			mfin[wave * 4 + i] = mrun[i];
+		}
 	}
 	__syncthreads();
 #pragma unroll
-	for (int a = 0; a < NACC; ++a) {
-		const int idx = tid + a * SEQ_THREADS;
-		if (idx < ATT_BR * rank) {
-			const int r = idx / rank, d = idx % rank;
-			if (r0 + r < NR)
-				Ctx[(size_t)(r0 + r) * rank + d] = acc[a] / lsum[r];
+	for (int a = 0; a < NA4; ++a) {
+		const int u = tid + a * SEQ_THREADS;
+		if (u < ATT_BR * q4n) {
+			const int r = u / q4n, d4 = u % q4n;
+			if (r0 + r >= NR)
+				continue;
+			if (S == 1) {
+				const float inv = 1.0f / lsum[r];
+#pragma unroll
+				for (int e = 0; e < 4; ++e)
+					if (4 * d4 + e < rank)
+						Ctx[(size_t)(r0 + r) * rank + 4 * d4 + e] = acc[a][e] * inv;
+			} else {
+				float *pp = part + ((size_t)(r0 + r) * S + split) * (rank4 + 4);
+				*(float4_t *)(pp + 4 * d4) = acc[a];
+				if (d4 == 0) {
+					pp[rank4] = mfin[r];
+					pp[rank4 + 1] = lsum[r];
+				}
+			}
 		}
 	}
 }
 static inline size_t att_lds_bytes(int rank) {
-	return sizeof(float) * ((size_t)ATT_BR * rank + (size_t)ATT_KT * (rank + 1) + ATT_BR * ATT_KT + 2 * ATT_BR);
+	const int r4 = att_rank4(rank);
+	return sizeof(float) * ((size_t)ATT_BR * r4 + (size_t)ATT_KT * (r4 + 4) + ATT_BR * ATT_KT + 3 * ATT_BR);
+}
+// Ctx[r] = sum_s e^(m_s - M) acc_s / sum_s e^(m_s - M) l_s over the key splits of row r.
+__global__ __launch_bounds__(64) void seq_latent_merge_kernel(const float *__restrict__ part, int S, int rank,
+                                                              float *__restrict__ Ctx) {
+	const int r = blockIdx.x, rank4 = att_rank4(rank), stride = rank4 + 4;
+	const float *pp = part + (size_t)r * S * stride;
+	float M = -FLT_MAX;
+	for (int s = 0; s < S; ++s)
+		M = fmaxf(M, pp[(size_t)s * stride + rank4]);
+	float L = 0.0f;
+	for (int s = 0; s < S; ++s)
+		L += expf(pp[(size_t)s * stride + rank4] - M) * pp[(size_t)s * stride + rank4 + 1];
+	const float inv = 1.0f / L;
+	for (int d = threadIdx.x; d < rank; d += 64) {
+		float v = 0.0f;
+		for (int s = 0; s < S; ++s)
+			v = fmaf(expf(pp[(size_t)s * stride + rank4] - M), pp[(size_t)s * stride + d], v);
+		Ctx[(size_t)r * rank + d] = v * inv;
+	}
 }
 
 // ------------------------------------------------------------------ routed experts
 // One workgroup per token: router logits in f32, softmax over all experts, a group's score
 // = its best expert's, only experts of the `keep` best groups can be chosen, the `top`
 // largest scores among them win (ties: the lower index); weight = score * rscale, not
-// renormalised. Also the shared expert's gate sigmoid(w_sg . h). Dynamic LDS: E floats.
+// renormalised. Also the shared expert's gate sigmoid(w_sg . h). Dynamic LDS: E + G floats.
 #define SEQ_MAX_GROUPS 64
 __global__ __launch_bounds__(SEQ_THREADS) void seq_router_kernel(const float *__restrict__ Hn, int width,
                                                                  const float *__restrict__ Wr, int E, int top, int G,
@@ -958,26 +1078,35 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_router_kernel(const float *__
 		}
 	}
 	__syncthreads();
-	if (threadIdx.x != 0)
-		return;
+	float *gsc = sc + E; // [G]
+	__shared__ float red[SEQ_THREADS / 64];
 	float mx = -FLT_MAX;
-	for (int e = 0; e < E; ++e)
+	for (int e = threadIdx.x; e < E; e += SEQ_THREADS)
 		mx = fmaxf(mx, sc[e]);
+	mx = wave_max(mx);
+	if (lane == 0)
+		red[wave] = mx;
+	__syncthreads();
+	mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
 	float sum = 0.0f;
-	for (int e = 0; e < E; ++e) {
-		sc[e] = expf(sc[e] - mx);
-		sum += sc[e];
+	for (int e = threadIdx.x; e < E; e += SEQ_THREADS) {
+		const float v = expf(sc[e] - mx);
+		sc[e] = v;
+		sum += v;
 	}
+	sum = block_sum(sum, red);
 	const float inv = 1.0f / sum;
 	const int gs = E / G;
-	unsigned long long allowed = 0ull; // groups that may be chosen from (G <= 64)
-	float gsc[SEQ_MAX_GROUPS];
-	for (int g = 0; g < G; ++g) {
+	for (int g = threadIdx.x; g < G; g += SEQ_THREADS) {
 		float m = -1.0f;
 		for (int e = g * gs; e < (g + 1) * gs; ++e)
 			m = fmaxf(m, sc[e]);
 		gsc[g] = m;
 	}
+	__syncthreads();
+	if (threadIdx.x != 0)
+		return;
+	unsigned long long allowed = 0ull; // groups that may be chosen from (G <= 64)
 	for (int k = 0; k < keep; ++k) {
 		int best = -1;
 		float bv = -2.0f;
