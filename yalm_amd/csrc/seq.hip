@@ -483,11 +483,12 @@ static int mixer_delta(Seq *q, int li, int n) {
 	                                                        bg);
 	const dim3 g(cdiv(V, SEQ_THREADS / 8), H);
 	const int R = cdiv(D, 8);
-#define DELTA_LAUNCH(RR) seq_delta_kernel<RR><<<g, SEQ_THREADS, 0, q->stream>>>(qkv, cc, KH, D, H, V, bg, q->S[li], o, n)
-	if (R <= 4) DELTA_LAUNCH(4);
-	else if (R <= 8) DELTA_LAUNCH(8);
-	else if (R <= 16) DELTA_LAUNCH(16);
-	else DELTA_LAUNCH(32);
+#define DELTA_LAUNCH(RR, TC)                                                                                           \
+	seq_delta_kernel<RR, TC><<<g, SEQ_THREADS, 0, q->stream>>>(qkv, cc, KH, D, H, V, bg, q->S[li], o, n)
+	if (R <= 4) DELTA_LAUNCH(4, 16);
+	else if (R <= 8) DELTA_LAUNCH(8, 16);
+	else if (R <= 16) DELTA_LAUNCH(16, 16);
+	else DELTA_LAUNCH(32, 8);
 #undef DELTA_LAUNCH
 	seq_delta_out_kernel<<<n, SEQ_THREADS, 0, q->stream>>>(o, H, V, l.out_norm, c.norm_eps, q->Z, zin, gcol, on);
 	HIPCHK(hipGetLastError());

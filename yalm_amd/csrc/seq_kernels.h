@@ -750,84 +750,123 @@ __device__ __forceinline__ float sum8(float v) { // over aligned groups of 8 lan
 // of 8 lanes owns one column (each lane a contiguous slice of R dim entries, in registers)
 // and walks the portion's tokens in order:
 //   S *= g;  u = beta (v - S.k);  S += k u;  o = S.q
-// (the read-out after the write). The next token's operands are loaded while the current
-// one is applied. grid (ceil(vdim / 32), heads).
-template <int R>
+// (the read-out after the write). The workgroup's 32 columns share the head's k and q:
+// chunks of TC tokens are staged through two LDS buffers, the next chunk's global loads in
+// flight while the current chunk is applied. grid (ceil(vdim / 32), heads).
+template <int R, int TC>
 __global__ __launch_bounds__(SEQ_THREADS) void seq_delta_kernel(const float *__restrict__ QKV, int ldq, int KH, int D,
                                                                 int H, int V, const float *__restrict__ BG,
                                                                 float *__restrict__ state, float *__restrict__ O,
                                                                 int T) {
+	constexpr int DP = 8 * R;                      // padded key dimension
+	constexpr int NKQ = TC * 2 * DP / SEQ_THREADS; // staged k | q values per thread and chunk
+	constexpr int COLS = SEQ_THREADS / 8, NV = (TC * COLS + SEQ_THREADS - 1) / SEQ_THREADS;
+	__shared__ __attribute__((aligned(16))) float kq[2][TC][2 * DP];
+	__shared__ float vs[2][TC][COLS], bgs[2][TC][2];
+	const int tid = threadIdx.x;
 	const int h = blockIdx.y, kh = h / (H / KH);
-	const int col = blockIdx.x * (SEQ_THREADS / 8) + (threadIdx.x >> 3), sub = threadIdx.x & 7;
+	const int c0 = blockIdx.x * COLS, col = c0 + (tid >> 3), sub = tid & 7;
 	const bool live = col < V;
-	const int vc = live ? col : V - 1;
 	const int d0 = sub * R; // this lane's slice of the key dimension: d0 .. d0 + R - 1
 	float S[R];
 	float *sp = state + (size_t)h * D * V;
 #pragma unroll
 	for (int i = 0; i < R; ++i)
-		S[i] = (d0 + i < D) ? sp[(size_t)(d0 + i) * V + vc] : 0.0f;
-	const int qo = kh * D, ko = KH * D + kh * D, vo = 2 * KH * D + h * V + vc;
-	// 16-byte loads when every lane's slice is whole and aligned
-	const bool vec = R % 4 == 0 && D % R == 0 && ldq % 4 == 0 && qo % 4 == 0 && ko % 4 == 0 && (size_t)QKV % 16 == 0;
-	const bool inside = d0 + R <= D;
-	float kn[R], qn[R], vn, bn, gn;
-	auto load = [&](int t) {
-		const float *row = QKV + (size_t)t * ldq;
-		if (vec && inside) {
+		S[i] = (live && d0 + i < D) ? sp[(size_t)(d0 + i) * V + col] : 0.0f;
+	const int qo = kh * D, ko = KH * D + kh * D, vo = 2 * KH * D + h * V;
+	// a chunk of TC tokens: global -> registers (in flight while the previous chunk is applied) -> LDS
+	float rkq[NKQ], rv[NV], rbg = 0.0f;
+	auto fetch = [&](int t0) {
 #pragma unroll
-			for (int i = 0; i < R / 4; ++i) {
-				const float4_t k4 = *(const float4_t *)(row + ko + d0 + 4 * i), q4 = *(const float4_t *)(row + qo + d0 + 4 * i);
+		for (int i = 0; i < NKQ; ++i) {
+			const int idx = tid + i * SEQ_THREADS;
+			const int tt = idx / (2 * DP), e = idx % (2 * DP), d = e % DP;
+			const int t = t0 + tt;
+			rkq[i] = (t < T && d < D) ? QKV[(size_t)t * ldq + (e < DP ? ko : qo) + d] : 0.0f;
+		}
 #pragma unroll
-				for (int e = 0; e < 4; ++e) {
-					kn[4 * i + e] = k4[e];
-					qn[4 * i + e] = q4[e];
+		for (int i = 0; i < NV; ++i) {
+			const int idx = tid + i * SEQ_THREADS;
+			const int tt = idx / COLS, cc = idx % COLS, t = t0 + tt;
+			rv[i] = (tt < TC && t < T && c0 + cc < V) ? QKV[(size_t)t * ldq + vo + c0 + cc] : 0.0f;
+		}
+		if (tid < 2 * TC) {
+			const int t = t0 + (tid >> 1);
+			rbg = t < T ? BG[(size_t)t * 2 * H + (tid & 1) * H + h] : 0.0f;
+		}
+	};
+	auto stash = [&](int buf) {
+#pragma unroll
+		for (int i = 0; i < NKQ; ++i) {
+			const int idx = tid + i * SEQ_THREADS;
+			kq[buf][idx / (2 * DP)][idx % (2 * DP)] = rkq[i];
+		}
+#pragma unroll
+		for (int i = 0; i < NV; ++i) {
+			const int idx = tid + i * SEQ_THREADS;
+			if (idx < TC * COLS)
+				vs[buf][idx / COLS][idx % COLS] = rv[i];
+		}
+		if (tid < 2 * TC)
+			bgs[buf][tid >> 1][tid & 1] = rbg;
+	};
+	fetch(0);
+	stash(0);
+	__syncthreads();
+	int buf = 0;
+	for (int t0 = 0; t0 < T; t0 += TC) {
+		const bool more = t0 + TC < T;
+		if (more)
+			fetch(t0 + TC);
+		const int nt = min(TC, T - t0);
+		for (int tt = 0; tt < nt; ++tt) {
+			float k[R], q[R];
+			if constexpr (R % 4 == 0) {
+#pragma unroll
+				for (int i = 0; i < R / 4; ++i) {
+					const float4_t k4 = *(const float4_t *)&kq[buf][tt][d0 + 4 * i];
+					const float4_t q4 = *(const float4_t *)&kq[buf][tt][DP + d0 + 4 * i];
+#pragma unroll
+					for (int e = 0; e < 4; ++e) {
+						k[4 * i + e] = k4[e];
+						q[4 * i + e] = q4[e];
+					}
+				}
+			} else {
+#pragma unroll
+				for (int i = 0; i < R; ++i) {
+					k[i] = kq[buf][tt][d0 + i];
+					q[i] = kq[buf][tt][DP + d0 + i];
 				}
 			}
-		} else {
+			const float v = vs[buf][tt][tid >> 3], beta = bgs[buf][tt][0], g = bgs[buf][tt][1];
+			float dd0 = 0.0f, dd1 = 0.0f;
 #pragma unroll
 			for (int i = 0; i < R; ++i) {
-				kn[i] = d0 + i < D ? row[ko + d0 + i] : 0.0f;
-				qn[i] = d0 + i < D ? row[qo + d0 + i] : 0.0f;
+				S[i] *= g;
+				if (i & 1)
+					dd1 = fmaf(S[i], k[i], dd1);
+				else
+					dd0 = fmaf(S[i], k[i], dd0);
 			}
-		}
-		vn = row[vo];
-		bn = BG[(size_t)t * 2 * H + h];
-		gn = BG[(size_t)t * 2 * H + H + h];
-	};
-	load(0);
-	for (int t = 0; t < T; ++t) {
-		float k[R], q[R];
+			const float u = beta * (v - sum8(dd0 + dd1));
+			float o0 = 0.0f, o1 = 0.0f;
 #pragma unroll
-		for (int i = 0; i < R; ++i) {
-			k[i] = kn[i];
-			q[i] = qn[i];
+			for (int i = 0; i < R; ++i) {
+				S[i] = fmaf(k[i], u, S[i]);
+				if (i & 1)
+					o1 = fmaf(S[i], q[i], o1);
+				else
+					o0 = fmaf(S[i], q[i], o0);
+			}
+			const float o = sum8(o0 + o1);
+			if (sub == 0 && live)
+				O[(size_t)(t0 + tt) * H * V + h * V + col] = o;
 		}
-		const float v = vn, beta = bn, g = gn;
-		if (t + 1 < T)
-			load(t + 1);
-		float dd0 = 0.0f, dd1 = 0.0f;
-#pragma unroll
-		for (int i = 0; i < R; ++i) {
-			S[i] *= g;
-			if (i & 1)
-				dd1 = fmaf(S[i], k[i], dd1);
-			else
-				dd0 = fmaf(S[i], k[i], dd0);
-		}
-		const float u = beta * (v - sum8(dd0 + dd1));
-		float o0 = 0.0f, o1 = 0.0f;
-#pragma unroll
-		for (int i = 0; i < R; ++i) {
-			S[i] = fmaf(k[i], u, S[i]);
-			if (i & 1)
-				o1 = fmaf(S[i], q[i], o1);
-			else
-				o0 = fmaf(S[i], q[i], o0);
-		}
-		const float o = sum8(o0 + o1);
-		if (sub == 0 && live)
-			O[(size_t)t * H * V + h * V + col] = o;
+		if (more)
+			stash(buf ^ 1); // last read while the chunk before this one was applied
+		__syncthreads();
+		buf ^= 1;
 	}
 	if (live) {
 #pragma unroll
@@ -1032,20 +1071,22 @@ static inline size_t att_lds_bytes(int rank) {
 // Ctx[r] = sum_s e^(m_s - M) acc_s / sum_s e^(m_s - M) l_s over the key splits of row r.
 __global__ __launch_bounds__(64) void seq_latent_merge_kernel(const float *__restrict__ part, int S, int rank,
                                                               float *__restrict__ Ctx) {
-	const int r = blockIdx.x, rank4 = att_rank4(rank), stride = rank4 + 4;
+	__shared__ float wsm[64]; // S <= 64: lane s holds split s
+	const int r = blockIdx.x, rank4 = att_rank4(rank), stride = rank4 + 4, lane = threadIdx.x;
 	const float *pp = part + (size_t)r * S * stride;
-	float M = -FLT_MAX;
-	for (int s = 0; s < S; ++s)
-		M = fmaxf(M, pp[(size_t)s * stride + rank4]);
-	float L = 0.0f;
-	for (int s = 0; s < S; ++s)
-		L += expf(pp[(size_t)s * stride + rank4] - M) * pp[(size_t)s * stride + rank4 + 1];
-	const float inv = 1.0f / L;
-	for (int d = threadIdx.x; d < rank; d += 64) {
+	const float m = lane < S ? pp[(size_t)lane * stride + rank4] : -FLT_MAX;
+	const float l = lane < S ? pp[(size_t)lane * stride + rank4 + 1] : 0.0f;
+	const float M = wave_max(m);
+	const float w = expf(m - M);
+	const float inv = 1.0f / wave_sum(w * l);
+	wsm[lane] = w * inv;
+	__syncthreads();
+	for (int d = lane; d < rank; d += 64) {
 		float v = 0.0f;
+#pragma unroll 4
 		for (int s = 0; s < S; ++s)
-			v = fmaf(expf(pp[(size_t)s * stride + rank4] - M), pp[(size_t)s * stride + d], v);
-		Ctx[(size_t)r * rank + d] = v * inv;
+			v = fmaf(wsm[s], pp[(size_t)s * stride + d], v);
+		Ctx[(size_t)r * rank + d] = v;
 	}
 }
 
@@ -1067,8 +1108,21 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_router_kernel(const float *__
 	for (int e = wave; e < E + (w_sg ? 1 : 0); e += SEQ_THREADS / 64) {
 		const float *w = e < E ? Wr + (size_t)e * width : w_sg;
 		float a = 0.0f;
-		for (int i = lane; i < width; i += 64)
-			a = fmaf(w[i], h[i], a);
+		if (width % 4 == 0 && ((size_t)w | (size_t)h) % 16 == 0) {
+			float a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+#pragma unroll 4
+			for (int i = lane * 4; i < width; i += 256) {
+				const float4_t wv = *(const float4_t *)(w + i), hv = *(const float4_t *)(h + i);
+				a = fmaf(wv[0], hv[0], a);
+				a1 = fmaf(wv[1], hv[1], a1);
+				a2 = fmaf(wv[2], hv[2], a2);
+				a3 = fmaf(wv[3], hv[3], a3);
+			}
+			a = (a + a1) + (a2 + a3);
+		} else {
+			for (int i = lane; i < width; i += 64)
+				a = fmaf(w[i], h[i], a);
+		}
 		a = wave_sum(a);
 		if (lane == 0) {
 			if (e < E)
