@@ -371,6 +371,20 @@ static GemmArgs plain(const float *A, int lda, const void *W, int ldw, float *C,
 template <class CT>
 static int attn_t(Seq *q, const float *Qa, const void *cache, int rank, int H, int n, float scale, float *ctx) {
 	const int NR = n * H;
+	if (sizeof(CT) == 2 && NR > 4 * ATT_BR) { // portions over a bf16 cache: the MFMA form
+		const dim3 gm(cdiv(NR, ATM_BR));
+		const int ks = cdiv(rank, 32);
+#define ATM_LAUNCH(KS)                                                                                                 \
+	seq_latent_attn_mfma_kernel<KS><<<gm, SEQ_THREADS, 0, q->stream>>>(Qa, (const uint16_t *)cache, rank, H, NR, scale,   \
+	                                                                  q->st, ctx)
+		if (ks <= 1) ATM_LAUNCH(1);
+		else if (ks <= 2) ATM_LAUNCH(2);
+		else if (ks <= 4) ATM_LAUNCH(4);
+		else ATM_LAUNCH(8);
+#undef ATM_LAUNCH
+		HIPCHK(hipGetLastError());
+		return YALM_OK;
+	}
 	// few rows (single tokens, short portions): the visible keys are split over workgroups
 	const int S = NR <= 4 * ATT_BR ? q->att_splits : 1;
 	const dim3 g(cdiv(NR, ATT_BR), S);

@@ -1090,6 +1090,146 @@ __global__ __launch_bounds__(64) void seq_latent_merge_kernel(const float *__res
 	}
 }
 
+// ---- portions over a bf16 cache: the same attention on the matrix cores. A workgroup owns
+// 64 rows (a wave 16) and walks the keys in tiles of 32; scores and weighted sums are
+// v_mfma_f32_16x16x32_bf16 products with f32 accumulation whose f32 operands (q~ * scale, the
+// softmax weights) enter as hi + lo bf16 pairs (hi = bf16(x), lo = bf16(x - hi): 16 significant
+// bits), the cached latent being bf16 already. Maximum, exponentials, running sums and the
+// rescaling of the sums stay f32, in the MFMA's C layout (row = 4 (lane >> 4) + reg, column =
+// lane & 15), where a row's 16 columns are the 16 lanes of a DPP row. KS = ceil(rank / 32).
+typedef float f32x4a_t __attribute__((ext_vector_type(4)));
+#define ATM_BR 64
+#define ATM_KT 32
+template <int KS>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_latent_attn_mfma_kernel(const float *__restrict__ Qa,
+                                                                           const uint16_t *__restrict__ cache, int rank,
+                                                                           int H, int NR, float scale,
+                                                                           const StepState *__restrict__ st,
+                                                                           float *__restrict__ Ctx) {
+	constexpr int R32 = 32 * KS, NT = 2 * KS; // padded rank, 16-wide output tiles
+	constexpr int LDC = R32 + 8, LDT = ATM_KT + 8, LDP = ATM_KT + 8;
+	__shared__ __attribute__((aligned(16))) uint16_t Cs[ATM_KT * LDC]; // [key][latent entry]
+	__shared__ __attribute__((aligned(16))) uint16_t CsT[R32 * LDT];   // [latent entry][key]
+	__shared__ __attribute__((aligned(16))) uint16_t Ps[4][2][16 * LDP]; // per wave: weights hi / lo [row][key]
+	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+	const int lr = lane & 15, lq = lane >> 4;
+	const int r0 = blockIdx.x * ATM_BR;
+	const int pos0 = st->pos;
+	const int rlast = min(r0 + ATM_BR, NR) - 1;
+	const int nkeys = pos0 + rlast / H + 1;
+	// this lane's A-operand row of q~ (row lr of the wave), as hi / lo fragments per 32-deep step
+	bf16x8_t qh[KS], ql[KS];
+	{
+		const int r = r0 + wave * 16 + lr;
+#pragma unroll
+		for (int sst = 0; sst < KS; ++sst) {
+			u32x4_t hi = {0, 0, 0, 0}, lo = {0, 0, 0, 0};
+#pragma unroll
+			for (int e = 0; e < 8; ++e) {
+				const int d = 32 * sst + 8 * lq + e;
+				const float x = (r < NR && d < rank) ? Qa[(size_t)r * rank + d] * scale : 0.0f;
+				const uint16_t hb = f2bf(x);
+				const uint16_t lb = f2bf(x - bf2f(hb));
+				hi[e >> 1] |= (uint32_t)hb << (16 * (e & 1));
+				lo[e >> 1] |= (uint32_t)lb << (16 * (e & 1));
+			}
+			qh[sst] = __builtin_bit_cast(bf16x8_t, hi);
+			ql[sst] = __builtin_bit_cast(bf16x8_t, lo);
+		}
+	}
+	int lim[4];
+	float mrun[4], lrun[4];
+#pragma unroll
+	for (int g = 0; g < 4; ++g) {
+		const int r = r0 + wave * 16 + 4 * lq + g;
+		lim[g] = r < NR ? pos0 + r / H : -1;
+		mrun[g] = -FLT_MAX;
+		lrun[g] = 0.0f;
+	}
+	f32x4a_t oacc[NT];
+#pragma unroll
+	for (int n = 0; n < NT; ++n)
+		oacc[n] = f32x4a_t{0.0f, 0.0f, 0.0f, 0.0f};
+	const bool cvec = rank % 8 == 0 && (size_t)cache % 16 == 0;
+	for (int kt = 0; kt < nkeys; kt += ATM_KT) {
+		__syncthreads(); // the previous tile's products have read Cs / CsT / Ps
+		for (int v = tid; v < ATM_KT * (R32 / 8); v += SEQ_THREADS) {
+			const int jj = v / (R32 / 8), d8 = (v % (R32 / 8)) * 8, j = kt + jj;
+			u32x4_t w = {0, 0, 0, 0};
+			if (j < nkeys) {
+				const uint16_t *src = cache + (size_t)j * rank + d8;
+				if (cvec && d8 + 8 <= rank) {
+					w = load16(src);
+				} else {
+#pragma unroll
+					for (int e = 0; e < 8; ++e)
+						if (d8 + e < rank)
+							w[e >> 1] |= (uint32_t)src[e] << (16 * (e & 1));
+				}
+			}
+			*(u32x4_t *)(Cs + jj * LDC + d8) = w;
+#pragma unroll
+			for (int e = 0; e < 8; ++e)
+				CsT[(d8 + e) * LDT + jj] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+		}
+		__syncthreads();
+		f32x4a_t sacc[2] = {f32x4a_t{0.0f, 0.0f, 0.0f, 0.0f}, f32x4a_t{0.0f, 0.0f, 0.0f, 0.0f}};
+#pragma unroll
+		for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+			for (int sst = 0; sst < KS; ++sst) {
+				const bf16x8_t kb =
+				    __builtin_bit_cast(bf16x8_t, *(const u32x4_t *)(Cs + (16 * jt + lr) * LDC + 32 * sst + 8 * lq));
+				sacc[jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qh[sst], kb, sacc[jt], 0, 0, 0);
+				sacc[jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ql[sst], kb, sacc[jt], 0, 0, 0);
+			}
+		float al[4];
+#pragma unroll
+		for (int g = 0; g < 4; ++g) {
+			const bool v0 = kt + lr <= lim[g], v1 = kt + 16 + lr <= lim[g];
+			const float s0 = v0 ? sacc[0][g] : -FLT_MAX, s1 = v1 ? sacc[1][g] : -FLT_MAX;
+			const float mnew = fmaxf(mrun[g], row16_max(fmaxf(s0, s1)));
+			const float p0 = v0 ? expf(s0 - mnew) : 0.0f, p1 = v1 ? expf(s1 - mnew) : 0.0f;
+			al[g] = expf(mrun[g] - mnew);
+			lrun[g] = lrun[g] * al[g] + row16_sum(p0 + p1);
+			mrun[g] = mnew;
+			const int row = 4 * lq + g;
+			const uint16_t h0 = f2bf(p0), h1 = f2bf(p1);
+			Ps[wave][0][row * LDP + lr] = h0;
+			Ps[wave][0][row * LDP + 16 + lr] = h1;
+			Ps[wave][1][row * LDP + lr] = f2bf(p0 - bf2f(h0));
+			Ps[wave][1][row * LDP + 16 + lr] = f2bf(p1 - bf2f(h1));
+		}
+#pragma unroll
+		for (int n = 0; n < NT; ++n)
+#pragma unroll
+			for (int g = 0; g < 4; ++g)
+				oacc[n][g] *= al[g];
+		__syncthreads(); // the wave's weights are in LDS
+		const bf16x8_t ph = __builtin_bit_cast(bf16x8_t, *(const u32x4_t *)(&Ps[wave][0][lr * LDP + 8 * lq]));
+		const bf16x8_t pl = __builtin_bit_cast(bf16x8_t, *(const u32x4_t *)(&Ps[wave][1][lr * LDP + 8 * lq]));
+#pragma unroll
+		for (int n = 0; n < NT; ++n) {
+			const bf16x8_t cb = __builtin_bit_cast(bf16x8_t, *(const u32x4_t *)(CsT + (16 * n + lr) * LDT + 8 * lq));
+			oacc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ph, cb, oacc[n], 0, 0, 0);
+			oacc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pl, cb, oacc[n], 0, 0, 0);
+		}
+	}
+#pragma unroll
+	for (int g = 0; g < 4; ++g) {
+		const int r = r0 + wave * 16 + 4 * lq + g;
+		if (r >= NR)
+			continue;
+		const float inv = 1.0f / lrun[g];
+#pragma unroll
+		for (int n = 0; n < NT; ++n) {
+			const int d = 16 * n + lr;
+			if (d < rank)
+				Ctx[(size_t)r * rank + d] = oacc[n][g] * inv;
+		}
+	}
+}
+
 // ------------------------------------------------------------------ routed experts
 // One workgroup per token: router logits in f32, softmax over all experts, a group's score
 // = its best expert's, only experts of the `keep` best groups can be chosen, the `top`
