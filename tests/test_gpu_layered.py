@@ -304,6 +304,59 @@ def test_greedy_generation(rt):
         model.close()
 
 
+def test_prompt_longer_than_one_internal_portion(rt):
+    """A step of more tokens than the engine's work buffers hold (4096) is cut inside the
+    engine; asked rows on both sides of the cut come back in order."""
+    from yalm_amd import models as M
+
+    cfg = C.config([("rglru", C.rglru(width=24, blocks=3, conv=3), None),
+                    ("latent_attention", C.latent(heads=1, dim=8, vdim=8, kv_rank=16, q_rank=8, scale=0.35), None)],
+                   width=32, vocab=53)
+    model, dec, w = build(rt, cfg, M.F32, seed=16, max_tokens=4300)
+    try:
+        tok = C.tokens(cfg, 4200, 15)
+        want = [0, 5, 4094, 4095, 4096, 4097, 4150, 4199]
+        got = dec.step(tok, want)
+        assert dec.pos == len(tok)
+        ref = R.forward(cfg, w, tok)[want]
+        assert rel_err(got, ref).max() < F32_TOL
+    finally:
+        dec.close()
+        model.close()
+
+
+def test_greedy_graph_replays_match_eager_steps(rt):
+    """The greedy loop replays one captured token graph. Several generate calls with ordinary
+    (eager) steps and synchronisations between them: every replayed token equals the argmax of
+    an eager step of a second decoder fed the same tokens."""
+    from yalm_amd import models as M
+
+    cfg = C.MIXED
+    model, dec, w = build(rt, cfg, M.F32, seed=17)
+    eager = rt.SeqDecoder(model)
+    try:
+        prompt = C.tokens(cfg, 9, 16)
+        dec.step(prompt[:-1])
+        eager.step(prompt[:-1])
+        tok = prompt[-1]
+        for n in (3, 1, 6, 2):
+            gen = dec.generate_greedy(tok, n)
+            for g in gen:
+                lg = eager.step([tok], [0])[0]
+                assert int(np.argmax(lg)) == g
+                tok = g
+            extra = C.tokens(cfg, 2, 17 + n)  # eager work on both between the replays
+            a = dec.step(extra, [1])
+            b = eager.step(extra, [1])
+            assert np.array_equal(a, b)
+            tok = int(np.argmax(a[0]))
+        assert dec.pos == eager.pos
+    finally:
+        dec.close()
+        eager.close()
+        model.close()
+
+
 def test_sequence_cannot_pass_max_tokens(rt):
     from yalm_amd import models as M
 

@@ -48,6 +48,12 @@ struct yalm_seq_s {
 	int dump_n = 0;
 	int *gen_tokens = nullptr;
 	int gen_cap = 0;
+	// one greedy token (step, logits, argmax) as a static hipGraph: every position-dependent
+	// value is read from the device StepState, so the same graph serves every token; the host
+	// then pays one launch per token instead of one per kernel (the greedy loop is otherwise
+	// bound by the host's launch rate, not by the device)
+	hipGraph_t greedy_graph = nullptr;
+	hipGraphExec_t greedy_exec = nullptr;
 	std::vector<void *> allocs;
 };
 typedef yalm_seq_s Seq;
@@ -136,6 +142,10 @@ static int validate(const yalm_seq_config &c, const std::vector<yalm_seq_layer> 
 
 // ------------------------------------------------------------------ create / destroy
 static void destroy_seq(Seq *q) {
+	if (q->greedy_exec)
+		(void)hipGraphExecDestroy(q->greedy_exec);
+	if (q->greedy_graph)
+		(void)hipGraphDestroy(q->greedy_graph);
 	for (void *p : q->allocs)
 		(void)hipFree(p);
 	if (q->own_stream && q->stream)
@@ -410,16 +420,15 @@ static int mixer_latent(Seq *q, int li, int n) {
 	const int zin = in_rows(l), H = l.heads, D = l.dim, V = l.vdim, rk = l.kv_rank;
 	float *cq = q->B[0], *qh = q->B[1], *qa = q->B[2], *ctx = q->B[3];
 	TRY(gemm(q, plain(q->Hn, c.width, l.w_in, c.width, q->Z, zin, n, zin, c.width)));
-	seq_norm_kernel<float><<<n, SEQ_THREADS, 0, q->stream>>>(q->Z, zin, l.q_norm, c.norm_eps, l.q_rank, cq, l.q_rank,
-	                                                         nullptr, q->st, 0);
-	if (l.kv_from < 0) {
-		if (bf)
-			seq_norm_kernel<uint16_t><<<n, SEQ_THREADS, 0, q->stream>>>(q->Z + l.q_rank, zin, l.kv_norm, c.norm_eps, rk,
-			                                                            (uint16_t *)q->cache[li], rk, nullptr, q->st, 1);
-		else
-			seq_norm_kernel<float><<<n, SEQ_THREADS, 0, q->stream>>>(q->Z + l.q_rank, zin, l.kv_norm, c.norm_eps, rk,
-			                                                         (float *)q->cache[li], rk, nullptr, q->st, 1);
-	}
+	if (l.kv_from >= 0)
+		seq_norm_kernel<float><<<n, SEQ_THREADS, 0, q->stream>>>(q->Z, zin, l.q_norm, c.norm_eps, l.q_rank, cq, l.q_rank,
+		                                                         nullptr, q->st, 0);
+	else if (bf)
+		seq_norm2_kernel<uint16_t><<<dim3(n, 2), SEQ_THREADS, 0, q->stream>>>(q->Z, zin, l.q_rank, l.q_norm, cq, rk, l.kv_norm,
+		                                                                    (uint16_t *)q->cache[li], c.norm_eps, q->st);
+	else
+		seq_norm2_kernel<float><<<dim3(n, 2), SEQ_THREADS, 0, q->stream>>>(q->Z, zin, l.q_rank, l.q_norm, cq, rk, l.kv_norm,
+		                                                                 (float *)q->cache[li], c.norm_eps, q->st);
 	HIPCHK(hipGetLastError());
 	TRY(gemm(q, plain(cq, l.q_rank, l.w_uq, l.q_rank, qh, H * D, n, H * D, l.q_rank)));
 	{ // q~[h] = W_uk[h]^T q[h]: per head [n][dim] x [rank][dim]^T
@@ -443,10 +452,15 @@ static int mixer_latent(Seq *q, int li, int n) {
 
 static int conv_launch(Seq *q, const float *Z, int ldz, int col0, int C, int taps, const float *w, const float *bias,
                        int silu, float *state, float *out, int n) {
-	seq_conv_kernel<<<dim3(cdiv(C, SEQ_THREADS), n), SEQ_THREADS, 0, q->stream>>>(Z, ldz, col0, C, taps, w, bias, silu,
-	                                                                              state, out, C, n);
-	if (taps > 1)
-		seq_conv_state_kernel<<<cdiv(C, SEQ_THREADS), SEQ_THREADS, 0, q->stream>>>(Z, ldz, col0, C, taps, state, n);
+	if (n <= SEQ_CONV_STEP_T) {
+		seq_conv_step_kernel<<<cdiv(C, SEQ_THREADS), SEQ_THREADS, 0, q->stream>>>(Z, ldz, col0, C, taps, w, bias, silu, state,
+		                                                                          out, C, n);
+	} else {
+		seq_conv_kernel<<<dim3(cdiv(C, SEQ_THREADS), n), SEQ_THREADS, 0, q->stream>>>(Z, ldz, col0, C, taps, w, bias, silu,
+		                                                                              state, out, C, n);
+		if (taps > 1)
+			seq_conv_state_kernel<<<cdiv(C, SEQ_THREADS), SEQ_THREADS, 0, q->stream>>>(Z, ldz, col0, C, taps, state, n);
+	}
 	HIPCHK(hipGetLastError());
 	return YALM_OK;
 }
@@ -462,15 +476,19 @@ static int mixer_rglru(Seq *q, int li, int n) {
 		TRY(gemm(q, a));
 	}
 	TRY(conv_launch(q, q->Z, 2 * W, W, W, l.conv, l.conv_w, l.conv_b, 0, q->conv[li], u, n));
-	for (int g = 0; g < 2; ++g) { // block-diagonal gates in f32
-		GemmArgs a = plain(u, W, g ? l.gate_i : l.gate_a, bs, g ? ig : r, W, n, bs, bs);
+	{ // both block-diagonal gates in f32, one launch: batches [0, blocks) recurrence gate, the rest input gate
+		GemmArgs a = plain(u, W, l.gate_a, bs, r, W, n, bs, bs);
 		a.a_bs = bs;
 		a.w_bs = (long)bs * bs;
 		a.c_bs = bs;
-		a.bias = g ? l.gate_i_b : l.gate_a_b;
+		a.bias = l.gate_a_b;
 		a.bias_bs = bs;
 		a.epi = EPI_SIGMOID;
-		TRY(gemm(q, a, l.blocks, -1, true));
+		a.z_split = l.blocks;
+		a.W_b = l.gate_i;
+		a.C_b = ig;
+		a.bias_b = l.gate_i_b;
+		TRY(gemm(q, a, 2 * l.blocks, -1, true));
 	}
 	if (n <= GEMV_MAX_M) {
 		seq_rglru_scan_kernel<<<cdiv(W, SEQ_THREADS), SEQ_THREADS, 0, q->stream>>>(r, ig, u, W, q->Z, 2 * W, l.lam,
@@ -576,15 +594,14 @@ static int ff_moe(Seq *q, int li, int n) {
 		TRY(gemm(q, a));
 		TRY(gemm(q, plain(hs, l.shared_ff, l.ws_down, l.shared_ff, ys, c.width, n, c.width, l.shared_ff)));
 	}
-	seq_moe_combine_kernel<<<dim3(cdiv(c.width, SEQ_THREADS), n), SEQ_THREADS, 0, q->stream>>>(
-	    yx, q->wt, top, l.shared_ff > 0 ? ys : nullptr, q->sgate, c.width, q->Y);
-	HIPCHK(hipGetLastError());
-	return YALM_OK;
+	return YALM_OK; // the combine of yx (B[1]) and ys (B[3]) happens in the closing norm's launch (add_norm)
 }
 
-static int add_norm(Seq *q, const float *wb, const float *w_next, int n) {
-	seq_add_norm_kernel<<<n, SEQ_THREADS, q->c.width * sizeof(float), q->stream>>>(q->X, q->Y, wb, q->c.norm_eps,
-	                                                                               q->c.width, w_next, q->Hn);
+// moe: the layer's routed experts feed the norm (their combine happens inside it) instead of Y
+static int add_norm(Seq *q, const float *wb, const float *w_next, int n, const yalm_seq_layer *moe = nullptr) {
+	seq_add_norm_kernel<<<n, SEQ_THREADS, q->c.width * sizeof(float), q->stream>>>(
+	    q->X, q->Y, wb, q->c.norm_eps, q->c.width, w_next, q->Hn, moe ? q->B[1] : nullptr, q->wt, moe ? moe->top : 0,
+	    moe && moe->shared_ff > 0 ? q->B[3] : nullptr, q->sgate);
 	HIPCHK(hipGetLastError());
 	return YALM_OK;
 }
@@ -596,12 +613,12 @@ static int enqueue_portion(Seq *q, const int *tokens_dev, int n) {
 	const yalm_seq_config &c = q->c;
 	if (c.weight_dtype == YALM_F32)
 		seq_embed_kernel<WF32><<<n, SEQ_THREADS, 0, q->stream>>>(q->st, tokens_dev, q->embed, q->inv_freq, c.width,
-		                                                         c.vocab, c.embed_scale, q->X);
+		                                                         c.vocab, c.embed_scale, q->X, q->L[0].norm1, c.norm_eps,
+		                                                         q->Hn);
 	else
 		seq_embed_kernel<WBF16><<<n, SEQ_THREADS, 0, q->stream>>>(q->st, tokens_dev, q->embed, q->inv_freq, c.width,
-		                                                          c.vocab, c.embed_scale, q->X);
-	seq_norm_kernel<float><<<n, SEQ_THREADS, 0, q->stream>>>(q->X, c.width, q->L[0].norm1, c.norm_eps, c.width, q->Hn,
-	                                                         c.width, nullptr, q->st, 0);
+		                                                          c.vocab, c.embed_scale, q->X, q->L[0].norm1, c.norm_eps,
+		                                                          q->Hn);
 	HIPCHK(hipGetLastError());
 	for (int li = 0; li < c.n_layers; ++li) {
 		const yalm_seq_layer &l = q->L[li];
@@ -617,7 +634,7 @@ static int enqueue_portion(Seq *q, const int *tokens_dev, int n) {
 		} else {
 			TRY(add_norm(q, l.norm1b, l.norm2, n));
 			TRY(l.ff_kind == YALM_FF_DENSE ? ff_dense(q, li, n) : ff_moe(q, li, n));
-			TRY(add_norm(q, l.norm2b, next, n));
+			TRY(add_norm(q, l.norm2b, next, n, l.ff_kind == YALM_FF_MOE ? &l : nullptr));
 		}
 		if (q->dump_on && q->dump)
 			HIPCHK(hipMemcpyAsync(q->dump + (size_t)li * n * c.width, q->X, (size_t)n * c.width * sizeof(float),
@@ -678,18 +695,44 @@ extern "C" int yalm_seq_step(yalm_seq q, const int *tokens, int n, const int *wa
 	return YALM_OK;
 }
 
+static int enqueue_greedy_token(Seq *q) {
+	TRY(enqueue_portion(q, nullptr, 1));
+	TRY(enqueue_logits(q, q->want, 1));
+	argmax_kernel<<<1, 1024, 0, q->stream>>>(q->logits, q->c.vocab, q->st, q->gen_tokens, q->gen_cap);
+	HIPCHK(hipGetLastError());
+	return YALM_OK;
+}
+
+static int ensure_greedy_graph(Seq *q) {
+	if (q->greedy_exec)
+		return YALM_OK;
+	HIPCHK(hipStreamBeginCapture(q->stream, hipStreamCaptureModeRelaxed));
+	const int r = enqueue_greedy_token(q);
+	hipGraph_t g = nullptr;
+	const hipError_t e = hipStreamEndCapture(q->stream, &g);
+	if (r != YALM_OK)
+		return r;
+	HIPCHK(e);
+	q->greedy_graph = g;
+	HIPCHK(hipGraphInstantiate(&q->greedy_exec, g, nullptr, nullptr, 0));
+	return YALM_OK;
+}
+
 extern "C" int yalm_seq_generate_greedy(yalm_seq q, int token, int n_steps, int *out_tokens) {
 	ARGCHK(q && out_tokens && n_steps > 0 && n_steps <= q->gen_cap, "yalm_seq_generate_greedy: bad argument");
 	ARGCHK(q->host_pos + n_steps <= q->c.max_tokens, "yalm_seq_generate_greedy: the sequence would pass max_tokens");
 	ARGCHK(token >= 0 && token < q->c.vocab, "yalm_seq_generate_greedy: token out of range");
+	const bool graph = !q->dump_on; // the layer dump's copies stay out of the graph
+	if (graph)
+		TRY(ensure_greedy_graph(q));
 	set_step_kernel<<<1, 1, 0, q->stream>>>(q->st, token, q->host_pos, 1);
 	seq_fill_int_kernel<<<1, 1, 0, q->stream>>>(q->want, 1, 0);
 	HIPCHK(hipGetLastError());
 	for (int i = 0; i < n_steps; ++i) {
-		TRY(enqueue_portion(q, nullptr, 1));
-		TRY(enqueue_logits(q, q->want, 1));
-		argmax_kernel<<<1, 1024, 0, q->stream>>>(q->logits, q->c.vocab, q->st, q->gen_tokens, q->gen_cap);
-		HIPCHK(hipGetLastError());
+		if (graph)
+			HIPCHK(hipGraphLaunch(q->greedy_exec, q->stream));
+		else
+			TRY(enqueue_greedy_token(q));
 	}
 	HIPCHK(hipMemcpyAsync(out_tokens, q->gen_tokens, (size_t)n_steps * sizeof(int), hipMemcpyDeviceToHost, q->stream));
 	HIPCHK(hipStreamSynchronize(q->stream));

@@ -65,16 +65,27 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_embed_kernel(const StepState 
                                                                 const int *__restrict__ tokens,
                                                                 const void *__restrict__ emb,
                                                                 const float *__restrict__ inv_freq, int width,
-                                                                int vocab, float scale, float *__restrict__ X) {
+                                                                int vocab, float scale, float *__restrict__ X,
+                                                                const float *__restrict__ w_next, float eps,
+                                                                float *__restrict__ Hn) {
+	__shared__ float red[SEQ_THREADS / 64];
 	const int t = blockIdx.x;
 	int tok = tokens ? tokens[t] : st->token;
 	tok = min(max(tok, 0), vocab - 1);
 	const float p = (float)(st->pos + t);
+	float ss = 0.0f;
 	for (int i = threadIdx.x; i < width; i += SEQ_THREADS) {
 		const float ang = p * inv_freq[i >> 1];
 		const float pe = (i & 1) ? cosf(ang) : sinf(ang);
-		X[(size_t)t * width + i] = wload<WT>(emb, (size_t)tok * width + i) * scale + pe;
+		const float v = wload<WT>(emb, (size_t)tok * width + i) * scale + pe;
+		X[(size_t)t * width + i] = v;
+		ss = fmaf(v, v, ss);
 	}
+	// the first layer's opening norm in the same launch (each thread re-reads its own entries)
+	ss = block_sum(ss, red);
+	const float r = 1.0f / sqrtf(ss / (float)width + eps);
+	for (int i = threadIdx.x; i < width; i += SEQ_THREADS)
+		Hn[(size_t)t * width + i] = X[(size_t)t * width + i] * r * w_next[i];
 }
 
 // ------------------------------------------------------------------ norms
@@ -104,21 +115,67 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_norm_kernel(const float *__re
 	}
 }
 
+// Two row norms of the same rows in one launch (blockIdx.y picks the segment): the query
+// latent into a f32 buffer and the key/value latent into the cache at rows st->pos + t.
+template <class OT>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_norm2_kernel(const float *__restrict__ in, int ld_in, int n0,
+                                                                const float *__restrict__ w0, float *__restrict__ out0,
+                                                                int n1, const float *__restrict__ w1,
+                                                                OT *__restrict__ out1, float eps,
+                                                                const StepState *__restrict__ st) {
+	__shared__ float red[SEQ_THREADS / 64];
+	const int t = blockIdx.x, seg = blockIdx.y;
+	const int n = seg ? n1 : n0;
+	const float *x = in + (size_t)t * ld_in + (seg ? n0 : 0);
+	const float *w = seg ? w1 : w0;
+	float ss = 0.0f;
+	for (int i = threadIdx.x; i < n; i += SEQ_THREADS)
+		ss = fmaf(x[i], x[i], ss);
+	ss = block_sum(ss, red);
+	const float r = 1.0f / sqrtf(ss / (float)n + eps);
+	for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
+		const float v = x[i] * r * w[i];
+		if (!seg) {
+			out0[(size_t)t * n0 + i] = v;
+		} else {
+			OT *o = out1 + (size_t)(st->pos + t) * n1;
+			if constexpr (sizeof(OT) == 2)
+				o[i] = f2bf(v);
+			else
+				o[i] = v;
+		}
+	}
+}
+
 // The seam between two sublayers in one launch: X[t] += norm(Y[t]) * wb (the closing norm
 // of the sublayer that produced Y and the residual sum), then, if w_next, Hn[t] =
 // norm(X[t]) * w_next (the opening norm of the next sublayer). Dynamic LDS: n floats.
+// Yx != null: Y is not read; its row is the routed experts' combine sum_k wt[t][k] Yx[t top + k]
+// (+ sgate[t] Ys[t], the shared expert), summed in slot order.
 __global__ __launch_bounds__(SEQ_THREADS) void seq_add_norm_kernel(float *__restrict__ X, const float *__restrict__ Y,
                                                                    const float *__restrict__ wb, float eps, int n,
                                                                    const float *__restrict__ w_next,
-                                                                   float *__restrict__ Hn) {
+                                                                   float *__restrict__ Hn,
+                                                                   const float *__restrict__ Yx,
+                                                                   const float *__restrict__ wt, int top,
+                                                                   const float *__restrict__ Ys,
+                                                                   const float *__restrict__ sgate) {
 	extern __shared__ float row[];
 	__shared__ float red[SEQ_THREADS / 64];
 	const int t = blockIdx.x;
-	const float *y = Y + (size_t)t * n;
 	float *x = X + (size_t)t * n;
 	float ss = 0.0f;
 	for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
-		const float v = y[i];
+		float v;
+		if (Yx) {
+			v = 0.0f;
+			for (int k = 0; k < top; ++k)
+				v = fmaf(wt[(size_t)t * top + k], Yx[((size_t)t * top + k) * n + i], v);
+			if (Ys)
+				v = fmaf(sgate[t], Ys[(size_t)t * n + i], v);
+		} else {
+			v = Y[(size_t)t * n + i];
+		}
 		row[i] = v;
 		ss = fmaf(v, v, ss);
 	}
@@ -165,6 +222,12 @@ struct GemmArgs {
 	int c_dense = 0; // 1: C row = m, 0: C row = list entry
 	int epi = EPI_NONE;
 	float limit = 0.0f;
+	// batches z >= z_split (z_split > 0) are a second product over the same A batches:
+	// matrices W_b, results C_b, bias bias_b, batch index z - z_split
+	int z_split = 0;
+	const void *W_b = nullptr;
+	float *C_b = nullptr;
+	const float *bias_b = nullptr;
 };
 
 __device__ __forceinline__ float epi_apply(const GemmArgs &a, float v, float v2, float b) {
@@ -191,13 +254,17 @@ struct GemmBatch {
 template <class WT>
 __device__ __forceinline__ GemmBatch gemm_batch(const GemmArgs &a, int z) {
 	GemmBatch b;
+	const bool second = a.z_split > 0 && z >= a.z_split;
+	if (second)
+		z -= a.z_split;
 	const long za = a.a_zdiv > 0 ? z / a.a_zdiv : z;
 	b.A = a.A + za * a.a_bs;
 	const long zw = a.w_sel ? a.w_sel[z] : z;
-	b.W = (const char *)a.W + zw * a.w_bs * WT::BYTES;
+	b.W = (const char *)(second ? a.W_b : a.W) + zw * a.w_bs * WT::BYTES;
 	b.W2 = a.W2 ? (const char *)a.W2 + zw * a.w_bs * WT::BYTES : nullptr;
-	b.C = a.C + (long)z * a.c_bs;
-	b.bias = a.bias ? a.bias + (long)z * a.bias_bs : nullptr;
+	b.C = (second ? a.C_b : a.C) + (long)z * a.c_bs;
+	const float *bias = second ? a.bias_b : a.bias;
+	b.bias = bias ? bias + (long)z * a.bias_bs : nullptr;
 	b.rows = a.rows ? a.rows + (long)z * a.rows_bs : nullptr;
 	b.M = a.counts ? a.counts[z] : a.M;
 	return b;
@@ -605,6 +672,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_gemm_bf16_kernel(GemmArgs a) 
 }
 
 // ------------------------------------------------------------------ short causal convolution
+#define SEQ_MAX_TAPS 16
 // out[t][c] = act(bias[c] + sum_j w[c][j] in(t - (taps - 1) + j)), in(tau) = Z[tau][col0 + c] for
 // tau >= 0, else the sequence's stored last inputs state[(taps - 1) + tau][c] (zeros at the start).
 __global__ __launch_bounds__(SEQ_THREADS) void seq_conv_kernel(const float *__restrict__ Z, int ldz, int col0, int C,
@@ -624,8 +692,46 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_conv_kernel(const float *__re
 	}
 	out[(size_t)t * ldo + c] = silu ? sq_silu(acc) : acc;
 }
+// Short portions (T <= SEQ_CONV_STEP_T): convolution and state shift in one launch, a thread
+// per channel walking the tokens with the last taps - 1 inputs in registers.
+#define SEQ_CONV_STEP_T 8
+__global__ __launch_bounds__(SEQ_THREADS) void seq_conv_step_kernel(const float *__restrict__ Z, int ldz, int col0, int C,
+                                                                    int taps, const float *__restrict__ w,
+                                                                    const float *__restrict__ bias, int silu,
+                                                                    float *__restrict__ state, float *__restrict__ out,
+                                                                    int ldo, int T) {
+	const int c = blockIdx.x * SEQ_THREADS + threadIdx.x;
+	if (c >= C)
+		return;
+	float win[SEQ_MAX_TAPS], wv[SEQ_MAX_TAPS]; // win[j]: input at (current token) - (taps - 1) + j
+#pragma unroll
+	for (int j = 0; j < SEQ_MAX_TAPS; ++j) {
+		win[j] = (j < taps - 1) ? state[(size_t)j * C + c] : 0.0f;
+		wv[j] = j < taps ? w[(size_t)c * taps + j] : 0.0f;
+	}
+	const float b = bias ? bias[c] : 0.0f;
+	for (int t = 0; t < T; ++t) {
+		const float cur = Z[(size_t)t * ldz + col0 + c];
+		float acc = b;
+#pragma unroll
+		for (int j = 0; j < SEQ_MAX_TAPS; ++j) {
+			if (j < taps) {
+				const float v = (j == taps - 1) ? cur : win[j];
+				acc = fmaf(wv[j], v, acc);
+			}
+		}
+		out[(size_t)t * ldo + c] = silu ? sq_silu(acc) : acc;
+#pragma unroll
+		for (int j = 0; j < SEQ_MAX_TAPS - 1; ++j) // shift the window by one token
+			if (j < taps - 1)
+				win[j] = (j + 1 < taps - 1) ? win[j + 1] : cur;
+	}
+#pragma unroll
+	for (int j = 0; j < SEQ_MAX_TAPS; ++j)
+		if (j < taps - 1)
+			state[(size_t)j * C + c] = win[j];
+}
 // The stored inputs after a portion of T tokens: the last taps - 1 of (old state ++ Z rows).
-#define SEQ_MAX_TAPS 16
 __global__ __launch_bounds__(SEQ_THREADS) void seq_conv_state_kernel(const float *__restrict__ Z, int ldz, int col0,
                                                                      int C, int taps, float *__restrict__ state,
                                                                      int T) {
@@ -1345,22 +1451,4 @@ __global__ void seq_fill_int_kernel(int *p, int n, int v) {
 __global__ void seq_fill_float_kernel(float *p, size_t n, float v) {
 	for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
 		p[i] = v;
-}
-
-// Y[t] = sum_k wt[t][k] Yx[t * top + k] (+ sgate[t] * Ys[t]).
-__global__ __launch_bounds__(SEQ_THREADS) void seq_moe_combine_kernel(const float *__restrict__ Yx,
-                                                                      const float *__restrict__ wt, int top,
-                                                                      const float *__restrict__ Ys,
-                                                                      const float *__restrict__ sgate, int width,
-                                                                      float *__restrict__ Y) {
-	const int t = blockIdx.y;
-	const int n = blockIdx.x * SEQ_THREADS + threadIdx.x;
-	if (n >= width)
-		return;
-	float v = 0.0f;
-	for (int k = 0; k < top; ++k)
-		v = fmaf(wt[(size_t)t * top + k], Yx[((size_t)t * top + k) * width + n], v);
-	if (Ys)
-		v = fmaf(sgate[t], Ys[(size_t)t * width + n], v);
-	Y[(size_t)t * width + n] = v;
 }

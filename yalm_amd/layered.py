@@ -162,7 +162,8 @@ def sinulorn_config(cfg: dict, max_tokens: int = 4096, weight_dtype: int = M.BF1
         elif kind == MIX_RGLRU:
             s = LayerSpec(kind, rec_width=m["width"], blocks=m["blocks"], conv=m["conv"])
         else:
-            s = LayerSpec(kind, heads=m["heads"], kv_heads=m["kv_heads"], dim=m["dim"], vdim=m["vdim"], conv=m["conv"])
+            s = LayerSpec(kind, heads=m["heads"], kv_heads=m.get("kv_heads", m["heads"]), dim=m["dim"], vdim=m["vdim"],
+                          conv=m["conv"])
         mlp = e.get("mlp")
         if mlp:
             if mlp["kind"] == "dense":
@@ -209,7 +210,7 @@ def sinulorn_tensor_shapes(cfg: dict) -> dict:
                 out[x + n], out[x + n + ".b"] = (B, R // B, R // B), (B, R // B)
             out[x + "lam"], out[x + "o"] = (R,), (W, R)
         else:
-            H, KH, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            H, KH, D, V = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m["vdim"]
             for n, rows in (("q", KH * D), ("k", KH * D), ("v", H * V)):
                 out[x + n], out[x + n + ".conv"] = (rows, W), (rows, m["conv"])
             out[x + "b"] = out[x + "a"] = (H, W)
