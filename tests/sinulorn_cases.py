@@ -70,5 +70,14 @@ WIDE = config([
 ], width=160, vocab=300)
 
 
+# sizes that are multiples of the large-tile GEMM's tiles (N % 128, K % 64): long portions of
+# this model run their plain products there when the whole library is loaded
+TILED = config([
+    ("rglru", rglru(width=256, blocks=4, conv=4), dense(ff=512)),
+    ("latent_attention", latent(heads=2, dim=64, vdim=64, kv_rank=64, q_rank=128, scale=0.11), dense(ff=384)),
+    ("delta", delta(heads=2, kv_heads=1, dim=64, vdim=64, conv=3), None),
+], width=256, vocab=384)
+
+
 def tokens(cfg, n, seed=0):
     return np.random.default_rng(1000 + seed).integers(0, cfg["vocab"], n).tolist()

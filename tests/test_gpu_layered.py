@@ -173,6 +173,26 @@ def test_bf16_stack_without_routing_is_strict(rt):
         model.close()
 
 
+def test_large_tile_products_bf16(rt):
+    """Tile-aligned sizes and a portion of more than 256 tokens: the plain products (input and
+    output projections with and without bias, the feed-forward's down projection, the head)
+    take the prefill unit's large-tile GEMM in its bf16 instantiation; shorter portions and
+    single tokens of the same sequence take the general kernels."""
+    from yalm_amd import models as M
+
+    cfg = C.TILED
+    model, dec, w = build(rt, cfg, M.BF16, seed=18, max_tokens=700)
+    try:
+        tok = C.tokens(cfg, 600, 18)
+        ref = R.forward(cfg, w, tok)
+        assert rel_err(dec.step(tok, list(range(len(tok)))), ref).max() < BF16_TOL
+        dec.reset()
+        assert rel_err(run_portions(dec, tok, [300, 5, 1, 1, 257, 20]), ref).max() < BF16_TOL
+    finally:
+        dec.close()
+        model.close()
+
+
 def test_portions_bf16_differ_by_rounding_only(rt):
     from yalm_amd import models as M
 

@@ -757,6 +757,26 @@ extern "C" int yalm_prefill_time(yalm_decoder d, int n, int iters, float *avg_ms
 	return YALM_OK;
 }
 
+// The layer-list engine's door to the large-tile GEMM (seq.hip; device pointers, asynchronous
+// on st): C [M][ldc] f32 = A [M][lda] bf16 . W [N][K]^T bf16 (+ bias[n]). Same tiles, phases
+// and tile-width choice as the f16 prefill GEMMs; YALM_ERR_UNSUPPORTED (nothing launched)
+// when the shape does not fit them: K % 64, no tile width dividing N, rows not 16-byte aligned.
+int pf_gemm_bf16(const uint16_t *A, int lda, int M, int K, const uint16_t *W, int N, float *C, int ldc,
+                 const float *bias, hipStream_t st) {
+	static const PfForms f = pf_forms_default();
+	if (M <= 0 || K % pf::BK != 0 || lda % 8 != 0 || ((size_t)A | (size_t)W) % 16 != 0)
+		return YALM_ERR_UNSUPPORTED;
+	const int bn = pick_bn(f, PG_TEST, M, N, false);
+	if (!bn)
+		return YALM_ERR_UNSUPPORTED;
+	pf::E16StoreF32B e;
+	e.c = C;
+	e.bias = bias;
+	e.ldc = ldc;
+	e.M = M;
+	return launch_plain(f, bn, A, lda, M, K, K, one(W, N), N, e, st);
+}
+
 extern "C" int yalm_gemm_f16(float *c, const uint16_t *a, const uint16_t *w, int M, int N, int K) {
 	ARGCHK(c && a && w && M > 0 && N > 0 && K > 0, "yalm_gemm_f16: bad argument");
 	ARGCHK(N % pf::BN == 0 && K % pf::BK == 0, "yalm_gemm_f16: N % 128 and K % 64 must be 0");

@@ -31,6 +31,8 @@
 // C layout (column = lane & 15, row = 4 (lane >> 4) + reg).
 #pragma once
 
+#include <type_traits>
+
 #include "prefill.h"
 
 namespace pf {
@@ -41,6 +43,24 @@ constexpr int G_BM = 256, G_BK = 64, G_THREADS = 512;
 
 // C/D map of v_mfma_f32_16x16x32: column = lane & 15, row = 4 (lane >> 4) + reg.
 __device__ __forceinline__ int crow16(int reg, int lane) { return 4 * (lane >> 4) + reg; }
+
+// Operand type of a GEMM instantiation: f16, or bf16 when the epilogue type says so
+// (static constexpr bool BF16 = true). The kernels move 16-bit words and never interpret
+// them outside this one product, so the bf16 GEMM of the layer-list engine is the same
+// code with the other MFMA.
+template <class EPI, class = void>
+struct epi_bf16 : std::false_type {};
+template <class EPI>
+struct epi_bf16<EPI, std::void_t<decltype(EPI::BF16)>> : std::bool_constant<EPI::BF16> {};
+typedef __bf16 bf16x8_pf_t __attribute__((ext_vector_type(8)));
+template <bool BF>
+__device__ __forceinline__ f32x4_t mfma16(const half8_t &a, const half8_t &b, const f32x4_t &c) {
+	if constexpr (BF)
+		return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_pf_t, a),
+		                                               __builtin_bit_cast(bf16x8_pf_t, b), c, 0, 0, 0);
+	else
+		return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
 
 // ---------------------------------------------------------------- B row policies
 struct BRowsPlain { // W rows n0 + r from up to 3 row-major [rows][K] matrices laid end to end
@@ -90,6 +110,32 @@ struct E16StoreF32 {
 				for (int j = 0; j < FJ; ++j)
 					c[(size_t)m * ldc + n0 + 16 * j + (lane & 15)] = acc[i][j][r];
 			}
+	}
+};
+
+// bf16 operands (epi_bf16), C[m][n] = acc (+ bias[n]) in f32: the layer-list engine's plain products
+struct E16StoreF32B {
+	static constexpr bool NEEDS_LDS = false;
+	static constexpr bool BF16 = true;
+	float *red = nullptr;
+	float *c;
+	const float *bias;
+	int ldc, M;
+	template <int FI, int FJ>
+	__device__ __forceinline__ void apply(f32x4_t (&acc)[FI][FJ], int m0, int n0, int lane, int, int) const {
+#pragma unroll
+		for (int j = 0; j < FJ; ++j) {
+			const int n = n0 + 16 * j + (lane & 15);
+			const float b = bias ? bias[n] : 0.0f;
+#pragma unroll
+			for (int i = 0; i < FI; ++i)
+#pragma unroll
+				for (int r = 0; r < 4; ++r) {
+					const int m = m0 + 16 * i + crow16(r, lane);
+					if (m < M)
+						c[(size_t)m * ldc + n] = acc[i][j][r] + b;
+				}
+		}
 	}
 };
 
@@ -425,7 +471,7 @@ __global__ __launch_bounds__(G_THREADS, 1) void gemm16_kernel(const uint16_t *__
 			for (int i = 0; i < FI; ++i)
 #pragma unroll
 				for (int j = 0; j < FJ; ++j)
-					acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+					acc[i][j] = mfma16<epi_bf16<EPI>::value>(af[i], bf[j], acc[i][j]);
 			__builtin_amdgcn_s_setprio(0);
 		}
 		asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // tile kt + 1 landed (this thread's DMAs)
@@ -645,7 +691,7 @@ __global__ __launch_bounds__(G_THREADS, 1) void gemm8p_kernel(const uint16_t *__
 	#pragma unroll
 					for (int ks = 0; ks < 2; ++ks)
 						acc[4 * mh + i][j] =
-						    __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][ks], b0[j][ks], acc[4 * mh + i][j], 0, 0, 0);
+						    mfma16<epi_bf16<EPI>::value>(a[i][ks], b0[j][ks], acc[4 * mh + i][j]);
 		};
 		auto mfma_n1 = [&](int mh) {
 	#pragma unroll
@@ -655,7 +701,7 @@ __global__ __launch_bounds__(G_THREADS, 1) void gemm8p_kernel(const uint16_t *__
 	#pragma unroll
 					for (int ks = 0; ks < 2; ++ks)
 						acc[4 * mh + i][FJ0 + j] =
-						    __builtin_amdgcn_mfma_f32_16x16x32_f16(a[i][ks], b1[j][ks], acc[4 * mh + i][FJ0 + j], 0, 0, 0);
+						    mfma16<epi_bf16<EPI>::value>(a[i][ks], b1[j][ks], acc[4 * mh + i][FJ0 + j]);
 		};
 
 		for (int it = 0;; ++it) {

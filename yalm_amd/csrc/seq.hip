@@ -19,6 +19,12 @@
 #include "misc_kernels.h"
 #include "seq_kernels.h"
 
+// The large-tile 8-phase GEMM of the prefill unit (prefill.hip), bf16 instantiation. Weak: the
+// library built from the shim and this unit alone has no prefill unit, and every product then
+// runs on this unit's general-shape kernels.
+int pf_gemm_bf16(const uint16_t *A, int lda, int M, int K, const uint16_t *W, int N, float *C, int ldc,
+                 const float *bias, hipStream_t st) __attribute__((weak));
+
 struct yalm_seq_s {
 	yalm_seq_config c{};
 	std::vector<yalm_seq_layer> L;
@@ -33,6 +39,7 @@ struct yalm_seq_s {
 	int zw = 0;                  // floats per row of Z (the widest input projection)
 	float *X = nullptr, *Hn = nullptr, *Y = nullptr, *Z = nullptr, *B[4] = {};
 	float *inv_freq = nullptr;
+	uint16_t *a16 = nullptr;     // [cap][bw] bf16 copy of a product's activations (large-tile GEMM operand)
 	int *tok = nullptr, *want = nullptr;
 	float *logits = nullptr;     // [LOGIT_ROWS][vocab]
 	int *idx = nullptr, *counts = nullptr, *lists = nullptr;
@@ -234,6 +241,8 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 	STRY(sallocT(q, &q->Z, cap * zw));
 	for (int i = 0; i < 4; ++i)
 		STRY(sallocT(q, &q->B[i], cap * bw));
+	if (bf && pf_gemm_bf16)
+		STRY(sallocT(q, &q->a16, cap * bw));
 	STRY(sallocT(q, &q->tok, cap));
 	STRY(sallocT(q, &q->want, cap));
 	STRY(sallocT(q, &q->logits, (size_t)LOGIT_ROWS * c.vocab));
@@ -362,6 +371,17 @@ static int gemm(Seq *q, const GemmArgs &a, int batches = 1, int max_m = -1, bool
 		max_m = a.M;
 	if (f32w || q->c.weight_dtype == YALM_F32)
 		return gemm_t<WF32>(q, a, batches, max_m);
+	// plain products of long portions whose shape fits the large-tile GEMM of the prefill unit
+	if (q->a16 && batches == 1 && max_m >= 2 * GB_BM && !a.W2 && !a.rows && !a.w_sel && a.epi == EPI_NONE &&
+	    a.z_split == 0 && a.ldw == a.K && a.K % 64 == 0 && a.N % 128 == 0 && (size_t)a.W % 16 == 0) {
+		const size_t n8 = (size_t)a.M * (a.K / 8);
+		seq_to_bf16_kernel<<<(unsigned)std::min<size_t>((n8 + SEQ_THREADS - 1) / SEQ_THREADS, 4096), SEQ_THREADS, 0,
+		                     q->stream>>>(a.A, a.lda, a.M, a.K, q->a16);
+		HIPCHK(hipGetLastError());
+		const int rc = pf_gemm_bf16(q->a16, a.K, a.M, a.K, (const uint16_t *)a.W, a.N, a.C, a.ldc, a.bias, q->stream);
+		if (rc != YALM_ERR_UNSUPPORTED)
+			return rc;
+	}
 	return gemm_t<WBF16>(q, a, batches, max_m);
 }
 static GemmArgs plain(const float *A, int lda, const void *W, int ldw, float *C, int ldc, int M, int N, int K) {

@@ -524,6 +524,23 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_gemm_kernel(GemmArgs a) {
 	}
 }
 
+// A [M][lda] f32 -> out [M][K] bf16 (round to nearest even): the A operand of the large-tile
+// GEMM (prefill_gemm.h), which takes 16-bit activations. K % 8 == 0.
+__global__ __launch_bounds__(SEQ_THREADS) void seq_to_bf16_kernel(const float *__restrict__ A, int lda, int M, int K,
+                                                                  uint16_t *__restrict__ out) {
+	const int k8 = K >> 3;
+	const size_t n = (size_t)M * k8;
+	for (size_t i = (size_t)blockIdx.x * SEQ_THREADS + threadIdx.x; i < n; i += (size_t)gridDim.x * SEQ_THREADS) {
+		const int m = (int)(i / k8), k = (int)(i % k8) * 8;
+		const float *src = A + (size_t)m * lda + k;
+		u32x4_t w;
+#pragma unroll
+		for (int e = 0; e < 4; ++e)
+			w[e] = (uint32_t)f2bf(src[2 * e]) | ((uint32_t)f2bf(src[2 * e + 1]) << 16);
+		*(u32x4_t *)(out + (size_t)m * K + k) = w;
+	}
+}
+
 // ---- long portions, bf16: 128 x 128 output tiles, 4 waves of 64 x 64 (2 x 2 MFMA tiles of
 // 32 x 32), K in slabs of 32 through two LDS buffers: the next slab's global loads (and the
 // activations' f32 -> bf16 rounding) are issued before the current slab's 8 MFMAs per wave
