@@ -79,5 +79,11 @@ TILED = config([
 ], width=256, vocab=384)
 
 
+# one routed layer whose shared expert's gated pair is tile-aligned (the routed experts' row
+# lists stay on the general kernel); last layer, so a flipped routing tie touches one position
+TILED_MOE = config([("rglru", rglru(width=128, blocks=2, conv=2), moe(ff=64, limit=1.25, experts=8, top=2, groups=2,
+                                                                     keep=2, shared=(128, 0.9)))], width=256, vocab=256)
+
+
 def tokens(cfg, n, seed=0):
     return np.random.default_rng(1000 + seed).integers(0, cfg["vocab"], n).tolist()

@@ -193,6 +193,20 @@ def test_large_tile_products_bf16(rt):
         model.close()
 
 
+def test_large_tile_clamped_pair_bf16(rt):
+    """The shared expert's clamped gated pair through the large-tile GEMM."""
+    from yalm_amd import models as M
+
+    cfg = C.TILED_MOE
+    model, dec, w = build(rt, cfg, M.BF16, seed=19, max_tokens=400)
+    try:
+        tok = C.tokens(cfg, 320, 19)
+        assert close_enough(dec.step(tok, list(range(len(tok)))), R.forward(cfg, w, tok), "bf16", 0.95)
+    finally:
+        dec.close()
+        model.close()
+
+
 def test_portions_bf16_differ_by_rounding_only(rt):
     from yalm_amd import models as M
 

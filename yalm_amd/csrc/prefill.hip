@@ -777,6 +777,28 @@ int pf_gemm_bf16(const uint16_t *A, int lda, int M, int K, const uint16_t *W, in
 	return launch_plain(f, bn, A, lda, M, K, K, one(W, N), N, e, st);
 }
 
+// The same door for a gated pair: C [M][ldc] f32 = act(A Wg^T) (.) (A Wu^T) over `hidden` units
+// (mode / limit: E16GluB), the two matrices' rows interleaved per wave as in the f16 prefill.
+int pf_gemm_glu_bf16(const uint16_t *A, int lda, int M, int K, const uint16_t *Wg, const uint16_t *Wu, int hidden,
+                     float *C, int ldc, int mode, float limit, hipStream_t st) {
+	static const PfForms f = pf_forms_default();
+	if (M <= 0 || K % pf::BK != 0 || lda % 8 != 0 || ((size_t)A | (size_t)Wg | (size_t)Wu) % 16 != 0)
+		return YALM_ERR_UNSUPPORTED;
+	const int bn = pick_bn(f, PG_GLU, M, 2 * hidden, true);
+	pf::E16GluB e;
+	e.c = C;
+	e.ldc = ldc;
+	e.M = M;
+	e.mode = mode;
+	e.limit = limit;
+	pf::BRowsGlu<64> bm{Wg, Wu};
+	if (bn == 256)
+		return launch_g16_t<pf::E16GluB, pf::BRowsGlu<64>, 256, 2>(f, A, lda, M, K, K, bm, 2 * hidden, e, st);
+	if (bn == 128)
+		return launch_g16_t<pf::E16GluB, pf::BRowsGlu<64>, 128, 4>(f, A, lda, M, K, K, bm, 2 * hidden, e, st);
+	return YALM_ERR_UNSUPPORTED;
+}
+
 extern "C" int yalm_gemm_f16(float *c, const uint16_t *a, const uint16_t *w, int M, int N, int K) {
 	ARGCHK(c && a && w && M > 0 && N > 0 && K > 0, "yalm_gemm_f16: bad argument");
 	ARGCHK(N % pf::BN == 0 && K % pf::BK == 0, "yalm_gemm_f16: N % 128 and K % 64 must be 0");

@@ -139,6 +139,41 @@ struct E16StoreF32B {
 	}
 };
 
+// bf16 operands, the layer-list engine's gated pairs over BRowsGlu rows (gate columns j <
+// FJ / 2, up columns j + FJ / 2 of the same hidden units), C f32: mode 1 gelu_tanh(g) u;
+// mode 2 g' sigmoid(1.702 g') (u' + 1) with g' = min(g, limit), u' = clamp(u, +-limit).
+struct E16GluB {
+	static constexpr bool NEEDS_LDS = false;
+	static constexpr bool BF16 = true;
+	float *red = nullptr;
+	float *c;
+	int ldc, M, mode;
+	float limit;
+	template <int FI, int FJ>
+	__device__ __forceinline__ void apply(f32x4_t (&acc)[FI][FJ], int m0, int n0, int lane, int, int) const {
+#pragma unroll
+		for (int i = 0; i < FI; ++i)
+#pragma unroll
+			for (int r = 0; r < 4; ++r) {
+				const int m = m0 + 16 * i + crow16(r, lane);
+				if (m >= M)
+					continue;
+#pragma unroll
+				for (int j = 0; j < FJ / 2; ++j) {
+					const float g = acc[i][j][r], u = acc[i][j + FJ / 2][r];
+					float v;
+					if (mode == 1) {
+						v = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))) * u;
+					} else {
+						const float gc = fminf(g, limit), uc = fminf(fmaxf(u, -limit), limit);
+						v = gc / (1.0f + expf(-1.702f * gc)) * (uc + 1.0f);
+					}
+					c[(size_t)m * ldc + n0 + 16 * j + (lane & 15)] = v;
+				}
+			}
+	}
+};
+
 struct E16Residual { // X[m][n] += scale C  (fused_matmul_add_residuals, per row)
 	static constexpr bool NEEDS_LDS = false;
 	float *red = nullptr;

@@ -25,6 +25,9 @@
 int pf_gemm_bf16(const uint16_t *A, int lda, int M, int K, const uint16_t *W, int N, float *C, int ldc,
                  const float *bias, hipStream_t st) __attribute__((weak));
 
+int pf_gemm_glu_bf16(const uint16_t *A, int lda, int M, int K, const uint16_t *Wg, const uint16_t *Wu, int hidden,
+                     float *C, int ldc, int mode, float limit, hipStream_t st) __attribute__((weak));
+
 struct yalm_seq_s {
 	yalm_seq_config c{};
 	std::vector<yalm_seq_layer> L;
@@ -372,13 +375,17 @@ static int gemm(Seq *q, const GemmArgs &a, int batches = 1, int max_m = -1, bool
 	if (f32w || q->c.weight_dtype == YALM_F32)
 		return gemm_t<WF32>(q, a, batches, max_m);
 	// plain products of long portions whose shape fits the large-tile GEMM of the prefill unit
-	if (q->a16 && batches == 1 && max_m >= 2 * GB_BM && !a.W2 && !a.rows && !a.w_sel && a.epi == EPI_NONE &&
-	    a.z_split == 0 && a.ldw == a.K && a.K % 64 == 0 && a.N % 128 == 0 && (size_t)a.W % 16 == 0) {
+	const bool pair = a.W2 != nullptr && (a.epi == EPI_GLU_GELU || a.epi == EPI_GLU_CLAMP) && !a.bias;
+	if (q->a16 && batches == 1 && max_m >= 2 * GB_BM && !a.rows && !a.w_sel && a.z_split == 0 && a.ldw == a.K &&
+	    a.K % 64 == 0 && (pair ? a.N % 64 == 0 : (!a.W2 && a.epi == EPI_NONE && a.N % 128 == 0))) {
 		const size_t n8 = (size_t)a.M * (a.K / 8);
 		seq_to_bf16_kernel<<<(unsigned)std::min<size_t>((n8 + SEQ_THREADS - 1) / SEQ_THREADS, 4096), SEQ_THREADS, 0,
 		                     q->stream>>>(a.A, a.lda, a.M, a.K, q->a16);
 		HIPCHK(hipGetLastError());
-		const int rc = pf_gemm_bf16(q->a16, a.K, a.M, a.K, (const uint16_t *)a.W, a.N, a.C, a.ldc, a.bias, q->stream);
+		const int rc =
+		    pair ? pf_gemm_glu_bf16(q->a16, a.K, a.M, a.K, (const uint16_t *)a.W, (const uint16_t *)a.W2, a.N, a.C, a.ldc,
+		                            a.epi == EPI_GLU_GELU ? 1 : 2, a.limit, q->stream)
+		         : pf_gemm_bf16(q->a16, a.K, a.M, a.K, (const uint16_t *)a.W, a.N, a.C, a.ldc, a.bias, q->stream);
 		if (rc != YALM_ERR_UNSUPPORTED)
 			return rc;
 	}
