@@ -246,6 +246,28 @@ def test_decoder_reused_after_reset(rt):
         model.close()
 
 
+def test_two_live_sequences_do_not_mix(rt):
+    """Two decoders on one model, their steps interleaved: each equals its sequence alone."""
+    from yalm_amd import models as M
+
+    cfg = C.MIXED
+    model, d1, w = build(rt, cfg, M.F32, seed=20)
+    d2 = rt.SeqDecoder(model)
+    try:
+        a, b = C.tokens(cfg, 60, 20), C.tokens(cfg, 45, 21)
+        ga, gb, ia, ib = [], [], 0, 0
+        for sa, sb in ((20, 3), (1, 30), (9, 1), (30, 11)):
+            ga.append(d1.step(a[ia:ia + sa], list(range(sa))))
+            gb.append(d2.step(b[ib:ib + sb], list(range(sb))))
+            ia, ib = ia + sa, ib + sb
+        assert rel_err(np.concatenate(ga), R.forward(cfg, w, a)).max() < F32_TOL
+        assert rel_err(np.concatenate(gb), R.forward(cfg, w, b)).max() < F32_TOL
+    finally:
+        d1.close()
+        d2.close()
+        model.close()
+
+
 def test_far_keys_decide_the_output(rt):
     """Peaked attention over a long prompt. The restatement's own softmax weights name a
     late query whose winning key lies more than 200 positions back; changing THAT token must

@@ -626,9 +626,19 @@ static int ff_moe(Seq *q, int li, int n) {
 
 // moe: the layer's routed experts feed the norm (their combine happens inside it) instead of Y
 static int add_norm(Seq *q, const float *wb, const float *w_next, int n, const yalm_seq_layer *moe = nullptr) {
-	seq_add_norm_kernel<<<n, SEQ_THREADS, q->c.width * sizeof(float), q->stream>>>(
-	    q->X, q->Y, wb, q->c.norm_eps, q->c.width, w_next, q->Hn, moe ? q->B[1] : nullptr, q->wt, moe ? moe->top : 0,
-	    moe && moe->shared_ff > 0 ? q->B[3] : nullptr, q->sgate);
+	const int w = q->c.width;
+	if (!moe && w <= 16 * SEQ_THREADS) { // the row in registers
+#define AN_LAUNCH(E)                                                                                                   \
+	seq_add_norm_reg_kernel<E><<<n, SEQ_THREADS, 0, q->stream>>>(q->X, q->Y, wb, q->c.norm_eps, w, w_next, q->Hn)
+		if (w <= 4 * SEQ_THREADS) AN_LAUNCH(4);
+		else if (w <= 8 * SEQ_THREADS) AN_LAUNCH(8);
+		else AN_LAUNCH(16);
+#undef AN_LAUNCH
+	} else {
+		seq_add_norm_kernel<<<n, SEQ_THREADS, w * sizeof(float), q->stream>>>(
+		    q->X, q->Y, wb, q->c.norm_eps, w, w_next, q->Hn, moe ? q->B[1] : nullptr, q->wt, moe ? moe->top : 0,
+		    moe && moe->shared_ff > 0 ? q->B[3] : nullptr, q->sgate);
+	}
 	HIPCHK(hipGetLastError());
 	return YALM_OK;
 }

@@ -150,6 +150,55 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_norm2_kernel(const float *__r
 // The seam between two sublayers in one launch: X[t] += norm(Y[t]) * wb (the closing norm
 // of the sublayer that produced Y and the residual sum), then, if w_next, Hn[t] =
 // norm(X[t]) * w_next (the opening norm of the next sublayer). Dynamic LDS: n floats.
+// Rows of up to E * SEQ_THREADS entries without a combine: the row of Y, the row of X and both
+// weight vectors are loaded at once (one memory round trip instead of one per pass) and the
+// row lives in registers.
+template <int E>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_add_norm_reg_kernel(float *__restrict__ X,
+                                                                       const float *__restrict__ Y,
+                                                                       const float *__restrict__ wb, float eps, int n,
+                                                                       const float *__restrict__ w_next,
+                                                                       float *__restrict__ Hn) {
+	__shared__ float red[SEQ_THREADS / 64];
+	const int t = blockIdx.x;
+	float y[E], x[E], b[E], wn[E];
+#pragma unroll
+	for (int e = 0; e < E; ++e) {
+		const int i = threadIdx.x + e * SEQ_THREADS;
+		const bool in = i < n;
+		y[e] = in ? Y[(size_t)t * n + i] : 0.0f;
+		x[e] = in ? X[(size_t)t * n + i] : 0.0f;
+		b[e] = in ? wb[i] : 0.0f;
+		wn[e] = (in && w_next) ? w_next[i] : 0.0f;
+	}
+	float ss = 0.0f;
+#pragma unroll
+	for (int e = 0; e < E; ++e)
+		ss = fmaf(y[e], y[e], ss);
+	ss = block_sum(ss, red);
+	const float r = 1.0f / sqrtf(ss / (float)n + eps);
+	float s2 = 0.0f;
+#pragma unroll
+	for (int e = 0; e < E; ++e) {
+		const int i = threadIdx.x + e * SEQ_THREADS;
+		x[e] = x[e] + y[e] * r * b[e];
+		if (i < n) {
+			X[(size_t)t * n + i] = x[e];
+			s2 = fmaf(x[e], x[e], s2);
+		}
+	}
+	if (!w_next)
+		return;
+	s2 = block_sum(s2, red);
+	const float r2 = 1.0f / sqrtf(s2 / (float)n + eps);
+#pragma unroll
+	for (int e = 0; e < E; ++e) {
+		const int i = threadIdx.x + e * SEQ_THREADS;
+		if (i < n)
+			Hn[(size_t)t * n + i] = x[e] * r2 * wn[e];
+	}
+}
+
 // Yx != null: Y is not read; its row is the routed experts' combine sum_k wt[t][k] Yx[t top + k]
 // (+ sgate[t] Ys[t], the shared expert), summed in slot order.
 __global__ __launch_bounds__(SEQ_THREADS) void seq_add_norm_kernel(float *__restrict__ X, const float *__restrict__ Y,
@@ -1084,16 +1133,37 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_latent_attn_kernel(const floa
 	}
 	for (int kt = k_begin; kt < k_end; kt += ATT_KT) {
 		__syncthreads(); // the previous tile's sums have read cs / ps
-		for (int i = tid; i < ATT_KT * rank4; i += SEQ_THREADS) {
-			const int jj = i / rank4, d = i % rank4, j = kt + jj;
-			float v = 0.0f;
-			if (j < k_end && d < rank) {
-				if constexpr (sizeof(CT) == 2)
-					v = bf2f(cache[(size_t)j * rank + d]);
-				else
-					v = cache[(size_t)j * rank + d];
+		if (rank % 8 == 0 && (size_t)cache % 16 == 0) { // 8 latent entries per load
+			const int v8n = rank >> 3;
+			for (int i = tid; i < ATT_KT * v8n; i += SEQ_THREADS) {
+				const int jj = i / v8n, d = (i % v8n) * 8, j = kt + jj;
+				float4_t lo = {0.0f, 0.0f, 0.0f, 0.0f}, hi = {0.0f, 0.0f, 0.0f, 0.0f};
+				if (j < k_end) {
+					if constexpr (sizeof(CT) == 2) {
+						float f[8];
+						WBF16::unpack(load16(cache + (size_t)j * rank + d), f);
+						lo = float4_t{f[0], f[1], f[2], f[3]};
+						hi = float4_t{f[4], f[5], f[6], f[7]};
+					} else {
+						lo = *(const float4_t *)(cache + (size_t)j * rank + d);
+						hi = *(const float4_t *)(cache + (size_t)j * rank + d + 4);
+					}
+				}
+				*(float4_t *)(cs + jj * ldc + d) = lo;
+				*(float4_t *)(cs + jj * ldc + d + 4) = hi;
 			}
-			cs[jj * ldc + d] = v;
+		} else {
+			for (int i = tid; i < ATT_KT * rank4; i += SEQ_THREADS) {
+				const int jj = i / rank4, d = i % rank4, j = kt + jj;
+				float v = 0.0f;
+				if (j < k_end && d < rank) {
+					if constexpr (sizeof(CT) == 2)
+						v = bf2f(cache[(size_t)j * rank + d]);
+					else
+						v = cache[(size_t)j * rank + d];
+				}
+				cs[jj * ldc + d] = v;
+			}
 		}
 		__syncthreads();
 		{
