@@ -345,7 +345,58 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_gemv_kernel(GemmArgs a) {
 	constexpr int E = 8; // elements per lane and pass
 	const bool vec = (a.ldw % E == 0) && (((size_t)b.W | (size_t)(GLU ? b.W2 : b.W)) % 16 == 0) && (a.lda % 4 == 0) &&
 	                 ((size_t)b.A % 16 == 0);
-	for (int k0 = lane * E; k0 < a.K; k0 += 64 * E) {
+	int kbeg = lane * E;
+	if (M == 1 && vec && a.K % E == 0) {
+		// one token, whole aligned rows: four 512-element steps of the weight row (non-temporal:
+		// read once per token) and of the activation row in flight before the first FMA
+		constexpr int U = 4;
+		for (; kbeg + (U - 1) * 64 * E < a.K; kbeg += U * 64 * E) {
+			u32x4_t wv[U][WT::BYTES == 2 ? 1 : 2], wv2[U][WT::BYTES == 2 ? 1 : 2];
+			float4_t xv[U][2];
+#pragma unroll
+			for (int u = 0; u < U; ++u) {
+				const int k = kbeg + u * 64 * E;
+				if constexpr (WT::BYTES == 2) {
+					wv[u][0] = load_nt16(w + (size_t)k * 2);
+					if constexpr (GLU)
+						wv2[u][0] = load_nt16(w2 + (size_t)k * 2);
+				} else {
+					wv[u][0] = load_nt16(w + (size_t)k * 4);
+					wv[u][1] = load_nt16(w + (size_t)k * 4 + 16);
+					if constexpr (GLU) {
+						wv2[u][0] = load_nt16(w2 + (size_t)k * 4);
+						wv2[u][1] = load_nt16(w2 + (size_t)k * 4 + 16);
+					}
+				}
+				xv[u][0] = *(const float4_t *)(ar[0] + k);
+				xv[u][1] = *(const float4_t *)(ar[0] + k + 4);
+			}
+#pragma unroll
+			for (int u = 0; u < U; ++u) {
+				float wf[E], wf2[E];
+				if constexpr (WT::BYTES == 2) {
+					WT::unpack(wv[u][0], wf);
+					if constexpr (GLU)
+						WT::unpack(wv2[u][0], wf2);
+				} else {
+					WT::unpack(wv[u][0], wf);
+					WT::unpack(wv[u][1], wf + 4);
+					if constexpr (GLU) {
+						WT::unpack(wv2[u][0], wf2);
+						WT::unpack(wv2[u][1], wf2 + 4);
+					}
+				}
+#pragma unroll
+				for (int e = 0; e < E; ++e) {
+					const float x = xv[u][e >> 2][e & 3];
+					acc[0] = fmaf(wf[e], x, acc[0]);
+					if constexpr (GLU)
+						acc2[0] = fmaf(wf2[e], x, acc2[0]);
+				}
+			}
+		}
+	}
+	for (int k0 = kbeg; k0 < a.K; k0 += 64 * E) {
 		float wf[E], wf2[E];
 		const bool full = vec && k0 + E <= a.K;
 		if (full) {
