@@ -311,9 +311,12 @@ int yalm_set_prefill_forms(yalm_decoder d, const char *spec);
 /* ---------------- layer-list models: mixers and feed-forwards chosen per layer ----------------
  * A second decoder kind beside yalm_decoder, for designs whose layers differ from one
  * another: every layer names a token mixer (latent attention over a cached low-rank
- * key/value latent, a real-gated linear recurrence, a gated delta rule) and a
- * feed-forward (none, dense GLU, routed experts with an optional shared expert), each
- * with its own sizes and constants. Around every sublayer: x += norm_b(f(norm(x))).
+ * key/value latent, a real-gated linear recurrence, a gated delta rule, softmax attention
+ * over cached keys and values with a window or chunk mask) and a feed-forward (none, dense
+ * GLU, routed experts with an optional shared expert, a plain two-matrix one), each with
+ * its own sizes and constants. Around every sublayer: x += norm_b(f(norm(x))) (pre_norm = 1)
+ * or x += norm_b(f(x)) (pre_norm = 0); the norms are rms norms or mean-subtracting layer
+ * norms (norm_kind), both with a weight and no bias.
  * One yalm_seq holds ONE sequence: its position, the latent caches and the recurrent
  * and convolution states, all in HBM; yalm_seq_step appends tokens (a whole prompt, a
  * portion of one, or a single decoded token) from where the last call stopped, so the
@@ -322,26 +325,52 @@ int yalm_set_prefill_forms(yalm_decoder d, const char *spec);
  * matrices: YALM_BF16 (bf16 MFMA products with f32 accumulation for portions, bf16
  * weight-streaming GEMVs for single tokens) or YALM_F32 (true f32 products).
  * Matrices are row-major [out][in]. */
-enum { YALM_MIX_LATENT = 0, YALM_MIX_RGLRU = 1, YALM_MIX_DELTA = 2 };
-enum { YALM_FF_NONE = 0, YALM_FF_DENSE = 1, YALM_FF_MOE = 2 };
+enum { YALM_MIX_LATENT = 0, YALM_MIX_RGLRU = 1, YALM_MIX_DELTA = 2, YALM_MIX_ATTN = 3 };
+enum { YALM_FF_NONE = 0, YALM_FF_DENSE = 1, YALM_FF_MOE = 2, YALM_FF_PLAIN = 3 };
+enum { YALM_NORM_RMS = 0, YALM_NORM_LAYER = 1 };
+/* attn: which earlier positions j <= i a position i sees */
+enum { YALM_MASK_CAUSAL = 0, /* all of them */
+	   YALM_MASK_WINDOW = 1, /* i - j < mask_size */
+	   YALM_MASK_CHUNK = 2 /* floor(i / mask_size) == floor(j / mask_size), chunks counted from position 0 */ };
+/* attn: norm of queries and keys */
+enum { YALM_QK_NONE = 0,
+	   YALM_QK_HEAD_UNIT = 1, /* after the rotation, every head divided by its rms over dim, no weight */
+	   YALM_QK_WHOLE = 2 /* before the rotation, rms norm over the whole projection with weights q_norm / kv_norm */ };
 
 typedef struct yalm_seq_layer {
 	int mixer;                     /* YALM_MIX_* */
 	int heads, kv_heads, dim, vdim; /* latent: heads x dim queries / keys, vdim values; delta: kv_heads x dim
-	                                  queries / keys shared by heads / kv_heads value heads of vdim */
+	                                  queries / keys shared by heads / kv_heads value heads of vdim; attn: heads
+	                                  query heads of dim, kv_heads key (dim) / value (vdim) heads, query head h
+	                                  reads key/value head h / (heads / kv_heads) */
 	int kv_rank, q_rank, kv_from;  /* latent: ranks; kv_from >= 0: read that layer's latent cache (no own w_in rows) */
-	float attn_scale;              /* latent: score = q.k * attn_scale */
+	float attn_scale;              /* latent, attn: score = q.k * attn_scale */
 	int rec_width, blocks;         /* rglru: channels, diagonal gate blocks */
 	int conv;                      /* rglru, delta: taps of the causal per-channel convolution */
-	int ff_kind, ff;               /* YALM_FF_*; ff: hidden size (dense) or one expert's (moe) */
+	int ff_kind, ff;               /* YALM_FF_*; ff: hidden size (dense, plain) or one expert's (moe) */
 	int experts, top, groups, groups_keep; /* moe: top experts among the groups_keep best of `groups` groups */
 	float router_scale, limit;     /* moe: weight = softmax score * router_scale; expert clamp */
 	int shared_ff;                 /* moe: shared expert's hidden size, 0 = none */
 	float shared_limit;
+	/* attn */
+	int mask_kind, mask_size;      /* YALM_MASK_* and its size in positions */
+	int qk_norm;                   /* YALM_QK_* */
+	int v_norm;                    /* 1: every value head divided by its rms over vdim (no weight) before it is cached */
+	int sink;                      /* 1: the softmax has one more key of score 0 and no value (1 added to the denominator) */
+	int out_gate;                  /* 1: head h's output times sigmoid(w_g[h] . x); the heads gate rows close w_in */
+	int rot_dims, rot_orig;        /* rotary positions on the first rot_dims entries of every query / key head, pairs
+	                                  (2i, 2i + 1), frequency rot_base^(-2i / rot_dims); rot_orig: see rot_factor */
+	float rot_base;
+	float rot_factor, rot_fast, rot_slow; /* rot_factor > 0: frequencies rescaled between the pair that turns rot_fast
+	                                  times and the pair that turns rot_slow times within rot_orig positions (f / factor
+	                                  where slower, f where faster, a linear ramp between), cos and sin times
+	                                  0.1 ln(rot_factor) + 1 */
 	/* f32 vectors */
 	const float *norm1, *norm1b, *norm2, *norm2b; /* [width] each; norm2* unused without a feed-forward */
-	const float *q_norm, *kv_norm;  /* latent: [q_rank], [kv_rank] */
-	const float *in_bias;           /* rglru: [2 rec_width] (gate branch, recurrent branch) */
+	const float *q_norm, *kv_norm;  /* latent: [q_rank], [kv_rank]; attn with YALM_QK_WHOLE: [heads dim], [kv_heads dim] */
+	const float *in_bias;           /* rglru: [2 rec_width] (gate branch, recurrent branch); attn: [rows of w_in] or NULL */
+	const float *head_temp;         /* attn: [heads], score of head h times head_temp[h], or NULL */
+	const float *talk;              /* attn: [heads][heads], score_h <- sum_g talk[h][g] score_g before mask and softmax, or NULL */
 	const float *conv_w, *conv_b;   /* [channels][conv] (last column = current token); rglru bias [rec_width] */
 	const float *gate_a, *gate_a_b, *gate_i, *gate_i_b; /* rglru: [blocks][bs][bs], [rec_width] (bs = rec_width / blocks) */
 	const float *lam;               /* rglru: [rec_width] */
@@ -350,12 +379,14 @@ typedef struct yalm_seq_layer {
 	/* matrices of weight_dtype */
 	const void *w_in;  /* latent: [q_rank (+ kv_rank if own latent)][width] (query down, latent down);
 	                      rglru: [2 rec_width][width] (gate branch, recurrent branch);
-	                      delta: [2 kv_heads dim + 2 heads vdim + 2 heads][width] (q, k, v, output gate, beta, decay) */
+	                      delta: [2 kv_heads dim + 2 heads vdim + 2 heads][width] (q, k, v, output gate, beta, decay);
+	                      attn: [heads dim + kv_heads dim + kv_heads vdim (+ heads if out_gate)][width] (q, k, v, gate) */
 	const void *w_uq;  /* latent: [heads dim][q_rank] */
 	const void *w_ukt; /* latent: [heads][kv_rank][dim], the key up-projection transposed per head */
 	const void *w_uv;  /* latent: [heads vdim][kv_rank] */
 	const void *w_o;   /* [width][heads vdim | rec_width] */
-	const void *w_gate, *w_up, *w_down; /* dense: [ff][width] x2, [width][ff]; moe: the same per expert, stacked */
+	const void *w_gate, *w_up, *w_down; /* dense: [ff][width] x2, [width][ff]; moe: the same per expert, stacked;
+	                                       plain: w_down gelu(w_up x), no w_gate */
 	const void *ws_gate, *ws_up, *ws_down; /* moe shared expert */
 } yalm_seq_layer;
 
@@ -363,6 +394,10 @@ typedef struct yalm_seq_config {
 	int width, vocab, n_layers, max_tokens; /* max_tokens: positions one sequence may hold */
 	float embed_scale, norm_eps;
 	int weight_dtype; /* YALM_BF16 | YALM_F32 */
+	int norm_kind;    /* YALM_NORM_*: every norm of the model (sublayers, final) */
+	int pre_norm;     /* 1: a sublayer reads norm1 / norm2 of the stream; 0: it reads the stream itself (norm1 / norm2 unused) */
+	int pos_embed;    /* 1: the interleaved sin / cos position vector (frequencies 10000^(-2i / width)) is added to the embedding */
+	float logit_scale; /* logits = head . norm(x) * logit_scale */
 } yalm_seq_config;
 
 typedef struct yalm_seq_weights {

@@ -1,7 +1,8 @@
 // seq.hip — the layer-list engine of the C ABI (include/yalm_hip.h, "layer-list models"):
 // a decoder whose layers each name their token mixer (latent attention, real-gated linear
-// recurrence, gated delta rule) and feed-forward (dense GLU, routed experts), holding one
-// sequence's latent caches and recurrent / convolution states in HBM. One step function
+// recurrence, gated delta rule, softmax attention with a window or chunk mask) and
+// feed-forward (dense GLU, routed experts, plain), holding one sequence's latent and
+// key / value caches and recurrent / convolution states in HBM. One step function
 // serves whole prompts, portions of prompts and single decoded tokens; the device greedy
 // loop feeds the argmax back without a host round trip, as yalm_generate_greedy does.
 #include "../../include/yalm_hip.h"
@@ -18,6 +19,7 @@
 #include "device_common.h"
 #include "misc_kernels.h"
 #include "seq_kernels.h"
+#include "seq_attn.h"
 
 // The large-tile 8-phase GEMM of the prefill unit (prefill.hip), bf16 instantiation. Weak: the
 // library built from the shim and this unit alone has no prefill unit, and every product then
@@ -41,6 +43,8 @@ struct yalm_seq_s {
 	size_t bw = 0;               // floats per row of the work buffers B0..B3
 	int zw = 0;                  // floats per row of Z (the widest input projection)
 	float *X = nullptr, *Hn = nullptr, *Y = nullptr, *Z = nullptr, *B[4] = {};
+	const float *In = nullptr;   // what a sublayer reads: Hn (pre_norm) or X itself
+	bool ln = false;             // the model's norms are layer norms
 	float *inv_freq = nullptr;
 	uint16_t *a16 = nullptr;     // [cap][bw] bf16 copy of a product's activations (large-tile GEMM operand)
 	int *tok = nullptr, *want = nullptr;
@@ -51,7 +55,11 @@ struct yalm_seq_s {
 	int att_splits = 1;          // key splits of single-token / short-portion attention
 	float *arena = nullptr;      // every recurrent and convolution state of the sequence
 	size_t arena_floats = 0;
-	std::vector<void *> cache;   // per layer: [max_tokens][kv_rank] latent rows (own latent only)
+	std::vector<void *> cache;   // per layer: [max_tokens][kv_rank] latent rows (own latent only); attn: key rows
+	std::vector<void *> vcache;  // attn: [max_tokens][kv_heads vdim] value rows
+	std::vector<double *> rot_freq; // attn: [rot_dims / 2] rotary angle per position
+	std::vector<float> rot_mag;
+	std::vector<int> attn_splits; // attn: key splits of single tokens and short portions
 	std::vector<float *> S, conv;
 	float *dump = nullptr;
 	bool dump_on = false;
@@ -91,6 +99,7 @@ static int in_rows(const yalm_seq_layer &l) {
 	switch (l.mixer) {
 	case YALM_MIX_LATENT: return l.q_rank + (l.kv_from < 0 ? l.kv_rank : 0);
 	case YALM_MIX_RGLRU: return 2 * l.rec_width;
+	case YALM_MIX_ATTN: return l.heads * l.dim + l.kv_heads * (l.dim + l.vdim) + (l.out_gate ? l.heads : 0);
 	default: return 2 * l.kv_heads * l.dim + 2 * l.heads * l.vdim + 2 * l.heads;
 	}
 }
@@ -98,10 +107,11 @@ static int in_rows(const yalm_seq_layer &l) {
 static int validate(const yalm_seq_config &c, const std::vector<yalm_seq_layer> &L) {
 	ARGCHK(c.width > 0 && c.vocab > 0 && c.n_layers > 0 && c.max_tokens > 0, "yalm_seq_create: bad model sizes");
 	ARGCHK(c.weight_dtype == YALM_BF16 || c.weight_dtype == YALM_F32, "yalm_seq_create: weight_dtype must be bf16 or f32");
+	ARGCHK(c.norm_kind == YALM_NORM_RMS || c.norm_kind == YALM_NORM_LAYER, "yalm_seq_create: unknown norm kind");
 	for (int i = 0; i < c.n_layers; ++i) {
 		const yalm_seq_layer &l = L[i];
 		const std::string at = "yalm_seq_create: layer " + std::to_string(i) + ": ";
-		ARGCHK(l.norm1 && l.norm1b && l.w_in && l.w_o, at + "missing tensors");
+		ARGCHK((l.norm1 || !c.pre_norm) && l.norm1b && l.w_in && l.w_o, at + "missing tensors");
 		if (l.mixer == YALM_MIX_LATENT) {
 			ARGCHK(l.heads > 0 && l.dim > 0 && l.vdim > 0 && l.kv_rank > 0 && l.q_rank > 0, at + "bad latent attention sizes");
 			if (l.kv_rank > 256) {
@@ -130,17 +140,34 @@ static int validate(const yalm_seq_config &c, const std::vector<yalm_seq_layer> 
 			}
 			ARGCHK(l.conv >= 1 && l.conv <= SEQ_MAX_TAPS, at + "convolution taps out of range");
 			ARGCHK(l.conv_w && l.a_log && l.dt_bias && l.out_norm, at + "missing delta rule tensors");
+		} else if (l.mixer == YALM_MIX_ATTN) {
+			ARGCHK(l.heads > 0 && l.kv_heads > 0 && l.heads % l.kv_heads == 0 && l.dim > 0 && l.vdim > 0,
+			       at + "bad attention sizes");
+			if (l.dim > 256 || l.vdim > 256 || (size_t)l.heads * ((l.vdim + 3) / 4) > (size_t)SA_MAX_NA4 * SEQ_THREADS) {
+				set_err(at + "heads of more than 256 entries (or heads x vdim above 16384) are not implemented by the attention kernels");
+				return YALM_ERR_UNSUPPORTED;
+			}
+			ARGCHK(l.mask_kind == YALM_MASK_CAUSAL || ((l.mask_kind == YALM_MASK_WINDOW || l.mask_kind == YALM_MASK_CHUNK) && l.mask_size > 0),
+			       at + "bad attention mask");
+			ARGCHK(l.qk_norm == YALM_QK_NONE || l.qk_norm == YALM_QK_HEAD_UNIT || (l.qk_norm == YALM_QK_WHOLE && l.q_norm && l.kv_norm),
+			       at + "bad query / key norm");
+			ARGCHK(l.rot_dims >= 0 && l.rot_dims <= l.dim && l.rot_dims % 2 == 0 && (l.rot_dims == 0 || l.rot_base > 0.0f),
+			       at + "rotary sizes must be even and at most dim");
+			ARGCHK(!(l.rot_factor > 0.0f) || (l.rot_orig > 0 && l.rot_fast > 0.0f && l.rot_slow > 0.0f && l.rot_base != 1.0f),
+			       at + "bad rotary rescaling");
 		} else {
 			ARGCHK(false, at + "unknown mixer");
 		}
 		if (l.ff_kind == YALM_FF_DENSE) {
-			ARGCHK(l.ff > 0 && l.w_gate && l.w_up && l.w_down && l.norm2 && l.norm2b, at + "bad dense feed-forward");
+			ARGCHK(l.ff > 0 && l.w_gate && l.w_up && l.w_down && (l.norm2 || !c.pre_norm) && l.norm2b, at + "bad dense feed-forward");
+		} else if (l.ff_kind == YALM_FF_PLAIN) {
+			ARGCHK(l.ff > 0 && l.w_up && l.w_down && (l.norm2 || !c.pre_norm) && l.norm2b, at + "bad plain feed-forward");
 		} else if (l.ff_kind == YALM_FF_MOE) {
 			ARGCHK(l.ff > 0 && l.experts > 0 && l.top > 0 && l.top <= l.experts && l.groups > 0 &&
 			           l.groups <= SEQ_MAX_GROUPS && l.experts % l.groups == 0 && l.groups_keep > 0 &&
 			           l.groups_keep <= l.groups && l.top <= l.groups_keep * (l.experts / l.groups),
 			       at + "bad router sizes");
-			ARGCHK(l.router && l.w_gate && l.w_up && l.w_down && l.norm2 && l.norm2b, at + "missing expert tensors");
+			ARGCHK(l.router && l.w_gate && l.w_up && l.w_down && (l.norm2 || !c.pre_norm) && l.norm2b, at + "missing expert tensors");
 			if (l.shared_ff > 0)
 				ARGCHK(l.ws_gate && l.ws_up && l.ws_down && l.shared_sg, at + "missing shared expert tensors");
 		} else {
@@ -175,6 +202,35 @@ static int att_attr_ct(int rank) {
 	if (na <= 1) return att_attr<CT, 1>(rank);
 	if (na <= 2) return att_attr<CT, 2>(rank);
 	return att_attr<CT, 4>(rank);
+}
+
+// attn: the rotary angle per position of every rotated pair, in double. Pair i turns
+// base^(-2i / dims) radians per position; with a rescaling (rot_factor > 0) the pairs that
+// turn fewer than rot_slow times within rot_orig positions turn rot_factor times slower, those
+// that turn more than rot_fast times are left, a linear ramp over the pair index between, and
+// cos / sin are scaled by 0.1 ln(rot_factor) + 1.
+static int attn_setup(yalm_seq_s *q, int li) {
+	const yalm_seq_layer &l = q->L[li];
+	const int dims = l.rot_dims, half = dims / 2;
+	std::vector<double> f(std::max(half, 1), 0.0);
+	double mag = 1.0;
+	for (int i = 0; i < half; ++i)
+		f[i] = std::pow((double)l.rot_base, -2.0 * i / (double)dims);
+	if (l.rot_factor > 0.0f && half > 0) {
+		const double pi = 3.14159265358979323846;
+		auto turn = [&](double t) { return dims * std::log((double)l.rot_orig / (2.0 * pi * t)) / (2.0 * std::log((double)l.rot_base)); };
+		const double lo = std::max(std::floor(turn(l.rot_fast)), 0.0);
+		const double hi = std::min(std::ceil(turn(l.rot_slow)), (double)(dims - 1));
+		for (int i = 0; i < half; ++i) {
+			const double ramp = std::min(std::max((i - lo) / std::max(hi - lo, 0.001), 0.0), 1.0);
+			f[i] = f[i] / (double)l.rot_factor * ramp + f[i] * (1.0 - ramp);
+		}
+		mag = 0.1 * std::log((double)l.rot_factor) + 1.0;
+	}
+	q->rot_mag[li] = (float)mag;
+	TRY(sallocT(q, &q->rot_freq[li], f.size()));
+	HIPCHK(hipMemcpy(q->rot_freq[li], f.data(), f.size() * sizeof(double), hipMemcpyHostToDevice));
+	return YALM_OK;
 }
 
 static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, yalm_stream s, Seq **out) {
@@ -221,12 +277,14 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 		} else if (l.mixer == YALM_MIX_RGLRU) {
 			bw = std::max(bw, (size_t)l.rec_width);
 			arena += (size_t)l.rec_width + (size_t)(l.conv - 1) * l.rec_width;
+		} else if (l.mixer == YALM_MIX_ATTN) {
+			bw = std::max({bw, (size_t)l.heads * l.dim, (size_t)l.heads * l.vdim});
 		} else {
 			const size_t cc = 2 * (size_t)l.kv_heads * l.dim + (size_t)l.heads * l.vdim;
 			bw = std::max({bw, cc, (size_t)l.heads * l.vdim, (size_t)2 * l.heads});
 			arena += (size_t)l.heads * l.dim * l.vdim + (size_t)(l.conv - 1) * cc;
 		}
-		if (l.ff_kind == YALM_FF_DENSE)
+		if (l.ff_kind == YALM_FF_DENSE || l.ff_kind == YALM_FF_PLAIN)
 			bw = std::max(bw, (size_t)l.ff);
 		if (l.ff_kind == YALM_FF_MOE) {
 			bw = std::max({bw, (size_t)l.top * l.ff, (size_t)l.top * c.width, (size_t)l.shared_ff});
@@ -262,12 +320,25 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 				max_rank = std::max(max_rank, l.kv_rank);
 			}
 		q->att_splits = std::max(1, std::min(32, cdiv(c.max_tokens, 2 * ATT_KT)));
-		STRY(sallocT(q, &q->att_part, (size_t)(4 * ATT_BR + GEMV_MAX_M * max_h) * q->att_splits * (att_rank4(max_rank) + 4)));
+		size_t part = (size_t)(4 * ATT_BR + GEMV_MAX_M * max_h) * q->att_splits * (att_rank4(max_rank) + 4);
+		// attn: the keys a single token can see, split so that a workgroup walks about two tiles
+		q->attn_splits.assign(c.n_layers, 1);
+		for (int i = 0; i < c.n_layers; ++i) {
+			const yalm_seq_layer &l = q->L[i];
+			if (l.mixer != YALM_MIX_ATTN)
+				continue;
+			const int span = l.mask_kind == YALM_MASK_CAUSAL ? c.max_tokens : std::min(c.max_tokens, l.mask_size + GEMV_MAX_M);
+			q->attn_splits[i] = std::max(1, std::min(32, cdiv(span, 2 * SA_KT)));
+			part = std::max(part, (size_t)GEMV_MAX_M * l.heads * q->attn_splits[i] * (att_rank4(l.vdim) + 4));
+		}
+		STRY(sallocT(q, &q->att_part, part));
 	}
 	q->gen_cap = 1 << 16;
 	STRY(sallocT(q, &q->gen_tokens, q->gen_cap));
+	q->ln = c.norm_kind == YALM_NORM_LAYER;
+	q->In = c.pre_norm ? q->Hn : q->X;
 	// position frequencies 10000^(-2 i / width), evaluated in double
-	{
+	if (c.pos_embed) {
 		std::vector<float> f((c.width + 1) / 2);
 		for (int i = 0; i < (c.width + 1) / 2; ++i)
 			f[i] = (float)std::pow(10000.0, -2.0 * i / (double)c.width);
@@ -282,6 +353,9 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 	q->cache.assign(c.n_layers, nullptr);
 	q->S.assign(c.n_layers, nullptr);
 	q->conv.assign(c.n_layers, nullptr);
+	q->vcache.assign(c.n_layers, nullptr);
+	q->rot_freq.assign(c.n_layers, nullptr);
+	q->rot_mag.assign(c.n_layers, 1.0f);
 	size_t off = 0;
 	for (int i = 0; i < c.n_layers; ++i) {
 		const yalm_seq_layer &l = q->L[i];
@@ -289,6 +363,10 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 			if (l.kv_from < 0)
 				STRY(salloc(q, &q->cache[i], (size_t)c.max_tokens * l.kv_rank * (bf ? 2 : 4)));
 			STRY(bf ? att_attr_ct<uint16_t>(l.kv_rank) : att_attr_ct<float>(l.kv_rank));
+		} else if (l.mixer == YALM_MIX_ATTN) {
+			STRY(salloc(q, &q->cache[i], (size_t)c.max_tokens * l.kv_heads * l.dim * (bf ? 2 : 4)));
+			STRY(salloc(q, &q->vcache[i], (size_t)c.max_tokens * l.kv_heads * l.vdim * (bf ? 2 : 4)));
+			STRY(attn_setup(q, i));
 		} else if (l.mixer == YALM_MIX_RGLRU) {
 			q->S[i] = q->arena + off;
 			off += l.rec_width;
@@ -446,7 +524,7 @@ static int mixer_latent(Seq *q, int li, int n) {
 	const bool bf = c.weight_dtype == YALM_BF16;
 	const int zin = in_rows(l), H = l.heads, D = l.dim, V = l.vdim, rk = l.kv_rank;
 	float *cq = q->B[0], *qh = q->B[1], *qa = q->B[2], *ctx = q->B[3];
-	TRY(gemm(q, plain(q->Hn, c.width, l.w_in, c.width, q->Z, zin, n, zin, c.width)));
+	TRY(gemm(q, plain(q->In, c.width, l.w_in, c.width, q->Z, zin, n, zin, c.width)));
 	if (l.kv_from >= 0)
 		seq_norm_kernel<float><<<n, SEQ_THREADS, 0, q->stream>>>(q->Z, zin, l.q_norm, c.norm_eps, l.q_rank, cq, l.q_rank,
 		                                                         nullptr, q->st, 0);
@@ -498,7 +576,7 @@ static int mixer_rglru(Seq *q, int li, int n) {
 	const int W = l.rec_width, bs = W / l.blocks;
 	float *u = q->B[0], *r = q->B[1], *ig = q->B[2], *so = q->B[3];
 	{
-		GemmArgs a = plain(q->Hn, c.width, l.w_in, c.width, q->Z, 2 * W, n, 2 * W, c.width);
+		GemmArgs a = plain(q->In, c.width, l.w_in, c.width, q->Z, 2 * W, n, 2 * W, c.width);
 		a.bias = l.in_bias;
 		TRY(gemm(q, a));
 	}
@@ -536,7 +614,7 @@ static int mixer_delta(Seq *q, int li, int n) {
 	const int CQ = KH * D, CV = H * V, cc = 2 * CQ + CV, zin = in_rows(l);
 	const int gcol = cc, bcol = cc + CV, acol = bcol + H;
 	float *qkv = q->B[0], *bg = q->B[1], *o = q->B[2], *on = q->B[3];
-	TRY(gemm(q, plain(q->Hn, c.width, l.w_in, c.width, q->Z, zin, n, zin, c.width)));
+	TRY(gemm(q, plain(q->In, c.width, l.w_in, c.width, q->Z, zin, n, zin, c.width)));
 	TRY(conv_launch(q, q->Z, zin, 0, cc, l.conv, l.conv_w, nullptr, 1, q->conv[li], qkv, n));
 	seq_delta_prep_kernel<<<n, SEQ_THREADS, 0, q->stream>>>(qkv, cc, KH, D, q->Z, zin, bcol, acol, H, l.a_log, l.dt_bias,
 	                                                        bg);
@@ -554,10 +632,102 @@ static int mixer_delta(Seq *q, int li, int n) {
 	return gemm(q, plain(on, CV, l.w_o, CV, q->Y, c.width, n, c.width, CV));
 }
 
+template <class CT>
+static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q, const float *gate, float *ctx) {
+	const yalm_seq_layer &l = q->L[li];
+	const bool talk = a.talk != nullptr;
+	const int Hb = talk ? a.H : a.H / a.G, V4n = (a.V + 3) / 4;
+	const int TQ = std::max(1, std::min(32 / Hb, n));
+	const int R = TQ * Hb;
+	const int S = n <= GEMV_MAX_M ? q->attn_splits[li] : 1;
+	const dim3 g(cdiv(n, TQ), S, talk ? 1 : a.G);
+	const size_t lds = sa_lds_bytes(R, a.H, a.D, a.V, talk);
+	const int na = cdiv(R * V4n, SEQ_THREADS);
+	const CT *Kc = (const CT *)q->cache[li], *Vc = (const CT *)q->vcache[li];
+#define SA_LAUNCH(NA)                                                                                                  \
+	do {                                                                                                               \
+		static bool attr_set = false; /* the kernel may use more dynamic LDS than the default limit */               \
+		if (!attr_set) {                                                                                               \
+			HIPCHK(hipFuncSetAttribute((const void *)seq_attn_kernel<CT, NA>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+			                           160 * 1024 - 64));                                                              \
+			attr_set = true;                                                                                           \
+		}                                                                                                              \
+		seq_attn_kernel<CT, NA><<<g, SEQ_THREADS, lds, q->stream>>>(Q, Kc, Vc, a, n, TQ, q->st, S == 1 ? gate : nullptr, \
+		                                                            ctx, q->att_part);                                 \
+	} while (0)
+	if (na <= 1) SA_LAUNCH(1);
+	else if (na <= 2) SA_LAUNCH(2);
+	else if (na <= 4) SA_LAUNCH(4);
+	else if (na <= 8) SA_LAUNCH(8);
+	else SA_LAUNCH(16);
+#undef SA_LAUNCH
+	if (S > 1)
+		seq_latent_merge_kernel<<<n * a.H, 64, 0, q->stream>>>(q->att_part, S, a.V, ctx, gate);
+	HIPCHK(hipGetLastError());
+	(void)l;
+	return YALM_OK;
+}
+
+// Softmax attention over cached keys and values: one input projection (queries, keys, values,
+// output gates), then rotation / norms / cache write, the attention itself, the output projection.
+static int mixer_attn(Seq *q, int li, int n) {
+	const yalm_seq_layer &l = q->L[li];
+	const yalm_seq_config &c = q->c;
+	const bool bf = c.weight_dtype == YALM_BF16;
+	const int zin = in_rows(l), H = l.heads, V = l.vdim;
+	float *Q = q->B[0], *gate = q->B[1], *ctx = q->B[2];
+	{
+		GemmArgs g = plain(q->In, c.width, l.w_in, c.width, q->Z, zin, n, zin, c.width);
+		g.bias = l.in_bias;
+		TRY(gemm(q, g));
+	}
+	AttnArgs a;
+	a.H = H;
+	a.G = l.kv_heads;
+	a.D = l.dim;
+	a.V = V;
+	a.mask_kind = l.mask_kind;
+	a.mask_size = l.mask_size;
+	a.qk_norm = l.qk_norm;
+	a.v_norm = l.v_norm;
+	a.sink = l.sink;
+	a.out_gate = l.out_gate;
+	a.rot_dims = l.rot_dims;
+	a.rot_mag = q->rot_mag[li];
+	a.rot_freq = q->rot_freq[li];
+	a.scale = l.attn_scale;
+	a.q_w = l.q_norm;
+	a.k_w = l.kv_norm;
+	a.temp = l.head_temp;
+	a.talk = l.talk;
+	a.eps = c.norm_eps;
+	const size_t rot_lds = (size_t)std::max(l.rot_dims, 2) * sizeof(float);
+	if (bf)
+		seq_attn_prep_kernel<uint16_t><<<n, SEQ_THREADS, rot_lds, q->stream>>>(q->Z, zin, a, q->st, Q, (uint16_t *)q->cache[li],
+		                                                                     (uint16_t *)q->vcache[li], gate);
+	else
+		seq_attn_prep_kernel<float><<<n, SEQ_THREADS, rot_lds, q->stream>>>(q->Z, zin, a, q->st, Q, (float *)q->cache[li],
+		                                                                  (float *)q->vcache[li], gate);
+	HIPCHK(hipGetLastError());
+	const float *gp = l.out_gate ? gate : nullptr;
+	TRY(bf ? attn_core_t<uint16_t>(q, li, n, a, Q, gp, ctx) : attn_core_t<float>(q, li, n, a, Q, gp, ctx));
+	return gemm(q, plain(ctx, H * V, l.w_o, H * V, q->Y, c.width, n, c.width, H * V));
+}
+
+// w_down gelu(w_up x)
+static int ff_plain(Seq *q, int li, int n) {
+	const yalm_seq_layer &l = q->L[li];
+	const yalm_seq_config &c = q->c;
+	GemmArgs a = plain(q->In, c.width, l.w_up, c.width, q->B[0], l.ff, n, l.ff, c.width);
+	a.epi = EPI_GELU;
+	TRY(gemm(q, a));
+	return gemm(q, plain(q->B[0], l.ff, l.w_down, l.ff, q->Y, c.width, n, c.width, l.ff));
+}
+
 static int ff_dense(Seq *q, int li, int n) {
 	const yalm_seq_layer &l = q->L[li];
 	const yalm_seq_config &c = q->c;
-	GemmArgs a = plain(q->Hn, c.width, l.w_gate, c.width, q->B[0], l.ff, n, l.ff, c.width);
+	GemmArgs a = plain(q->In, c.width, l.w_gate, c.width, q->B[0], l.ff, n, l.ff, c.width);
 	a.W2 = l.w_up;
 	a.epi = EPI_GLU_GELU;
 	TRY(gemm(q, a));
@@ -569,13 +739,13 @@ static int ff_moe(Seq *q, int li, int n) {
 	const yalm_seq_config &c = q->c;
 	const int E = l.experts, top = l.top, ff = l.ff, slots = n * top;
 	float *hx = q->B[0], *yx = q->B[1], *hs = q->B[2], *ys = q->B[3];
-	seq_router_kernel<<<n, SEQ_THREADS, (E + l.groups) * sizeof(float), q->stream>>>(q->Hn, c.width, l.router, E, top, l.groups,
+	seq_router_kernel<<<n, SEQ_THREADS, (E + l.groups) * sizeof(float), q->stream>>>(q->In, c.width, l.router, E, top, l.groups,
 	                                                                    l.groups_keep, l.router_scale,
 	                                                                    l.shared_ff > 0 ? l.shared_sg : nullptr, q->idx,
 	                                                                    q->wt, q->sgate);
 	HIPCHK(hipGetLastError());
 	if (n <= GEMV_MAX_M) { // one batch per (token, choice): its expert's matrices picked on the device
-		GemmArgs a = plain(q->Hn, c.width, l.w_gate, c.width, hx, ff, 1, ff, c.width);
+		GemmArgs a = plain(q->In, c.width, l.w_gate, c.width, hx, ff, 1, ff, c.width);
 		a.W2 = l.w_up;
 		a.a_bs = c.width;
 		a.a_zdiv = top;
@@ -596,7 +766,7 @@ static int ff_moe(Seq *q, int li, int n) {
 		seq_moe_lists_kernel<<<cdiv(slots, SEQ_THREADS), SEQ_THREADS, 0, q->stream>>>(q->idx, slots, q->counts, q->lists,
 		                                                                              q->cap);
 		HIPCHK(hipGetLastError());
-		GemmArgs a = plain(q->Hn, c.width, l.w_gate, c.width, hx, ff, n, ff, c.width);
+		GemmArgs a = plain(q->In, c.width, l.w_gate, c.width, hx, ff, n, ff, c.width);
 		a.W2 = l.w_up;
 		a.w_bs = (long)ff * c.width;
 		a.rows = q->lists;
@@ -614,7 +784,7 @@ static int ff_moe(Seq *q, int li, int n) {
 		TRY(gemm(q, b, E, n));
 	}
 	if (l.shared_ff > 0) {
-		GemmArgs a = plain(q->Hn, c.width, l.ws_gate, c.width, hs, l.shared_ff, n, l.shared_ff, c.width);
+		GemmArgs a = plain(q->In, c.width, l.ws_gate, c.width, hs, l.shared_ff, n, l.shared_ff, c.width);
 		a.W2 = l.ws_up;
 		a.epi = EPI_GLU_CLAMP;
 		a.limit = l.shared_limit;
@@ -629,7 +799,7 @@ static int add_norm(Seq *q, const float *wb, const float *w_next, int n, const y
 	const int w = q->c.width;
 	if (!moe && w <= 16 * SEQ_THREADS) { // the row in registers
 #define AN_LAUNCH(E)                                                                                                   \
-	seq_add_norm_reg_kernel<E><<<n, SEQ_THREADS, 0, q->stream>>>(q->X, q->Y, wb, q->c.norm_eps, w, w_next, q->Hn)
+	seq_add_norm_reg_kernel<E><<<n, SEQ_THREADS, 0, q->stream>>>(q->X, q->Y, wb, q->c.norm_eps, w, w_next, q->Hn, (int)q->ln)
 		if (w <= 4 * SEQ_THREADS) AN_LAUNCH(4);
 		else if (w <= 8 * SEQ_THREADS) AN_LAUNCH(8);
 		else AN_LAUNCH(16);
@@ -637,7 +807,7 @@ static int add_norm(Seq *q, const float *wb, const float *w_next, int n, const y
 	} else {
 		seq_add_norm_kernel<<<n, SEQ_THREADS, w * sizeof(float), q->stream>>>(
 		    q->X, q->Y, wb, q->c.norm_eps, w, w_next, q->Hn, moe ? q->B[1] : nullptr, q->wt, moe ? moe->top : 0,
-		    moe && moe->shared_ff > 0 ? q->B[3] : nullptr, q->sgate);
+		    moe && moe->shared_ff > 0 ? q->B[3] : nullptr, q->sgate, (int)q->ln);
 	}
 	HIPCHK(hipGetLastError());
 	return YALM_OK;
@@ -648,29 +818,34 @@ static int add_norm(Seq *q, const float *wb, const float *w_next, int n, const y
 // position is st->pos on the device (set by the caller).
 static int enqueue_portion(Seq *q, const int *tokens_dev, int n) {
 	const yalm_seq_config &c = q->c;
+	const bool pre = c.pre_norm != 0; // else the sublayers read the stream itself and no opening norm is computed
+	const float *first_norm = pre ? q->L[0].norm1 : nullptr;
 	if (c.weight_dtype == YALM_F32)
 		seq_embed_kernel<WF32><<<n, SEQ_THREADS, 0, q->stream>>>(q->st, tokens_dev, q->embed, q->inv_freq, c.width,
-		                                                         c.vocab, c.embed_scale, q->X, q->L[0].norm1, c.norm_eps,
-		                                                         q->Hn);
+		                                                         c.vocab, c.embed_scale, q->X, first_norm, c.norm_eps,
+		                                                         q->Hn, (int)q->ln);
 	else
 		seq_embed_kernel<WBF16><<<n, SEQ_THREADS, 0, q->stream>>>(q->st, tokens_dev, q->embed, q->inv_freq, c.width,
-		                                                          c.vocab, c.embed_scale, q->X, q->L[0].norm1, c.norm_eps,
-		                                                          q->Hn);
+		                                                          c.vocab, c.embed_scale, q->X, first_norm, c.norm_eps,
+		                                                          q->Hn, (int)q->ln);
 	HIPCHK(hipGetLastError());
 	for (int li = 0; li < c.n_layers; ++li) {
 		const yalm_seq_layer &l = q->L[li];
-		const float *next = li + 1 < c.n_layers ? q->L[li + 1].norm1 : nullptr;
+		const float *next = pre && li + 1 < c.n_layers ? q->L[li + 1].norm1 : nullptr;
 		if (l.mixer == YALM_MIX_LATENT)
 			TRY(mixer_latent(q, li, n));
 		else if (l.mixer == YALM_MIX_RGLRU)
 			TRY(mixer_rglru(q, li, n));
+		else if (l.mixer == YALM_MIX_ATTN)
+			TRY(mixer_attn(q, li, n));
 		else
 			TRY(mixer_delta(q, li, n));
 		if (l.ff_kind == YALM_FF_NONE) {
 			TRY(add_norm(q, l.norm1b, next, n));
 		} else {
-			TRY(add_norm(q, l.norm1b, l.norm2, n));
-			TRY(l.ff_kind == YALM_FF_DENSE ? ff_dense(q, li, n) : ff_moe(q, li, n));
+			TRY(add_norm(q, l.norm1b, pre ? l.norm2 : nullptr, n));
+			TRY(l.ff_kind == YALM_FF_DENSE ? ff_dense(q, li, n)
+			                               : (l.ff_kind == YALM_FF_PLAIN ? ff_plain(q, li, n) : ff_moe(q, li, n)));
 			TRY(add_norm(q, l.norm2b, next, n, l.ff_kind == YALM_FF_MOE ? &l : nullptr));
 		}
 		if (q->dump_on && q->dump)
@@ -684,7 +859,8 @@ static int enqueue_portion(Seq *q, const int *tokens_dev, int n) {
 static int enqueue_logits(Seq *q, const int *rows_dev, int n_rows) {
 	const yalm_seq_config &c = q->c;
 	seq_norm_kernel<float><<<n_rows, SEQ_THREADS, 0, q->stream>>>(q->X, c.width, q->final_norm, c.norm_eps, c.width,
-	                                                              q->Hn, c.width, rows_dev, q->st, 0);
+	                                                              q->Hn, c.width, rows_dev, q->st, 0, (int)q->ln,
+	                                                              c.logit_scale);
 	HIPCHK(hipGetLastError());
 	return gemm(q, plain(q->Hn, c.width, q->head, c.width, q->logits, c.vocab, n_rows, c.vocab, c.width));
 }

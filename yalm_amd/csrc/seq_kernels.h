@@ -57,9 +57,16 @@ __device__ __forceinline__ float block_sum(float v, float *red) {
 	return t;
 }
 
+// The two norm kinds (YALM_NORM_*): an rms norm divides a row by sqrt(mean(x^2) + eps); a layer
+// norm first takes the row's mean off, then divides by sqrt(mean(deviation^2) + eps). Both are
+// followed by a weight and have no bias. Kernels take `ln` (1 = layer norm) and subtract the
+// mean from the entries they hold before the sum of squares (two passes over values already
+// in registers or LDS, so the variance is that of the deviations themselves).
+
 // ------------------------------------------------------------------ embedding
-// X[t] = embed[token] * scale + the interleaved (sin, cos) position vector of position
-// st->pos + t; tokens == nullptr: the single device-resident token of the greedy loop.
+// X[t] = embed[token] * scale (+ the interleaved (sin, cos) position vector of position
+// st->pos + t if inv_freq); tokens == nullptr: the single device-resident token of the greedy
+// loop. w_next != nullptr: also Hn[t] = norm(X[t]) * w_next, the first layer's opening norm.
 template <class WT>
 __global__ __launch_bounds__(SEQ_THREADS) void seq_embed_kernel(const StepState *__restrict__ st,
                                                                 const int *__restrict__ tokens,
@@ -67,47 +74,72 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_embed_kernel(const StepState 
                                                                 const float *__restrict__ inv_freq, int width,
                                                                 int vocab, float scale, float *__restrict__ X,
                                                                 const float *__restrict__ w_next, float eps,
-                                                                float *__restrict__ Hn) {
+                                                                float *__restrict__ Hn, int ln) {
 	__shared__ float red[SEQ_THREADS / 64];
 	const int t = blockIdx.x;
 	int tok = tokens ? tokens[t] : st->token;
 	tok = min(max(tok, 0), vocab - 1);
 	const float p = (float)(st->pos + t);
-	float ss = 0.0f;
+	float ss = 0.0f, sm = 0.0f;
 	for (int i = threadIdx.x; i < width; i += SEQ_THREADS) {
-		const float ang = p * inv_freq[i >> 1];
-		const float pe = (i & 1) ? cosf(ang) : sinf(ang);
+		float pe = 0.0f;
+		if (inv_freq) {
+			const float ang = p * inv_freq[i >> 1];
+			pe = (i & 1) ? cosf(ang) : sinf(ang);
+		}
 		const float v = wload<WT>(emb, (size_t)tok * width + i) * scale + pe;
 		X[(size_t)t * width + i] = v;
 		ss = fmaf(v, v, ss);
+		sm += v;
 	}
+	if (!w_next)
+		return;
 	// the first layer's opening norm in the same launch (each thread re-reads its own entries)
+	float mu = 0.0f;
+	if (ln) {
+		mu = block_sum(sm, red) / (float)width;
+		ss = 0.0f;
+		for (int i = threadIdx.x; i < width; i += SEQ_THREADS) {
+			const float d = X[(size_t)t * width + i] - mu;
+			ss = fmaf(d, d, ss);
+		}
+	}
 	ss = block_sum(ss, red);
 	const float r = 1.0f / sqrtf(ss / (float)width + eps);
 	for (int i = threadIdx.x; i < width; i += SEQ_THREADS)
-		Hn[(size_t)t * width + i] = X[(size_t)t * width + i] * r * w_next[i];
+		Hn[(size_t)t * width + i] = (X[(size_t)t * width + i] - mu) * r * w_next[i];
 }
 
 // ------------------------------------------------------------------ norms
-// out[row(t)] = in[t] / sqrt(mean(in[t]^2) + eps) * w, one workgroup per row. rows != null:
-// the input row is rows[t] (gather). pos_rows: the output row is st->pos + t (a cache write).
+// out[row(t)] = norm(in[t]) * w * post, one workgroup per row. rows != null: the input row
+// is rows[t] (gather). pos_rows: the output row is st->pos + t (a cache write).
 template <class OT>
 __global__ __launch_bounds__(SEQ_THREADS) void seq_norm_kernel(const float *__restrict__ in, int ld_in,
                                                                const float *__restrict__ w, float eps, int n,
                                                                OT *__restrict__ out, int ld_out,
                                                                const int *__restrict__ rows,
-                                                               const StepState *__restrict__ st, int pos_rows) {
+                                                               const StepState *__restrict__ st, int pos_rows,
+                                                               int ln = 0, float post = 1.0f) {
 	__shared__ float red[SEQ_THREADS / 64];
 	const int t = blockIdx.x;
 	const float *x = in + (size_t)(rows ? rows[t] : t) * ld_in;
+	float mu = 0.0f;
+	if (ln) {
+		float sm = 0.0f;
+		for (int i = threadIdx.x; i < n; i += SEQ_THREADS)
+			sm += x[i];
+		mu = block_sum(sm, red) / (float)n;
+	}
 	float ss = 0.0f;
-	for (int i = threadIdx.x; i < n; i += SEQ_THREADS)
-		ss = fmaf(x[i], x[i], ss);
+	for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
+		const float d = x[i] - mu;
+		ss = fmaf(d, d, ss);
+	}
 	ss = block_sum(ss, red);
-	const float r = 1.0f / sqrtf(ss / (float)n + eps);
+	const float r = post / sqrtf(ss / (float)n + eps);
 	OT *o = out + (size_t)(pos_rows ? st->pos + t : t) * ld_out;
 	for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
-		const float v = x[i] * r * w[i];
+		const float v = (x[i] - mu) * r * w[i];
 		if constexpr (sizeof(OT) == 2)
 			o[i] = f2bf(v);
 		else
@@ -158,7 +190,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_add_norm_reg_kernel(float *__
                                                                        const float *__restrict__ Y,
                                                                        const float *__restrict__ wb, float eps, int n,
                                                                        const float *__restrict__ w_next,
-                                                                       float *__restrict__ Hn) {
+                                                                       float *__restrict__ Hn, int ln) {
 	__shared__ float red[SEQ_THREADS / 64];
 	const int t = blockIdx.x;
 	float y[E], x[E], b[E], wn[E];
@@ -171,13 +203,24 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_add_norm_reg_kernel(float *__
 		b[e] = in ? wb[i] : 0.0f;
 		wn[e] = (in && w_next) ? w_next[i] : 0.0f;
 	}
+	if (ln) { // entries past the row's end stay 0
+		float sm = 0.0f;
+#pragma unroll
+		for (int e = 0; e < E; ++e)
+			sm += y[e];
+		const float mu = block_sum(sm, red) / (float)n;
+#pragma unroll
+		for (int e = 0; e < E; ++e)
+			if (threadIdx.x + e * SEQ_THREADS < n)
+				y[e] -= mu;
+	}
 	float ss = 0.0f;
 #pragma unroll
 	for (int e = 0; e < E; ++e)
 		ss = fmaf(y[e], y[e], ss);
 	ss = block_sum(ss, red);
 	const float r = 1.0f / sqrtf(ss / (float)n + eps);
-	float s2 = 0.0f;
+	float s2 = 0.0f, sm2 = 0.0f;
 #pragma unroll
 	for (int e = 0; e < E; ++e) {
 		const int i = threadIdx.x + e * SEQ_THREADS;
@@ -185,10 +228,21 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_add_norm_reg_kernel(float *__
 		if (i < n) {
 			X[(size_t)t * n + i] = x[e];
 			s2 = fmaf(x[e], x[e], s2);
+			sm2 += x[e];
 		}
 	}
 	if (!w_next)
 		return;
+	if (ln) {
+		const float mu = block_sum(sm2, red) / (float)n;
+		s2 = 0.0f;
+#pragma unroll
+		for (int e = 0; e < E; ++e)
+			if (threadIdx.x + e * SEQ_THREADS < n) {
+				x[e] -= mu;
+				s2 = fmaf(x[e], x[e], s2);
+			}
+	}
 	s2 = block_sum(s2, red);
 	const float r2 = 1.0f / sqrtf(s2 / (float)n + eps);
 #pragma unroll
@@ -208,12 +262,12 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_add_norm_kernel(float *__rest
                                                                    const float *__restrict__ Yx,
                                                                    const float *__restrict__ wt, int top,
                                                                    const float *__restrict__ Ys,
-                                                                   const float *__restrict__ sgate) {
+                                                                   const float *__restrict__ sgate, int ln) {
 	extern __shared__ float row[];
 	__shared__ float red[SEQ_THREADS / 64];
 	const int t = blockIdx.x;
 	float *x = X + (size_t)t * n;
-	float ss = 0.0f;
+	float ss = 0.0f, sm = 0.0f;
 	for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
 		float v;
 		if (Yx) {
@@ -227,26 +281,46 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_add_norm_kernel(float *__rest
 		}
 		row[i] = v;
 		ss = fmaf(v, v, ss);
+		sm += v;
+	}
+	float mu = 0.0f;
+	if (ln) { // each thread re-reads the entries it wrote
+		mu = block_sum(sm, red) / (float)n;
+		ss = 0.0f;
+		for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
+			const float d = row[i] - mu;
+			ss = fmaf(d, d, ss);
+		}
 	}
 	ss = block_sum(ss, red);
 	const float r = 1.0f / sqrtf(ss / (float)n + eps);
-	float s2 = 0.0f;
+	float s2 = 0.0f, sm2 = 0.0f;
 	for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
-		const float v = x[i] + row[i] * r * wb[i];
+		const float v = x[i] + (row[i] - mu) * r * wb[i];
 		x[i] = v;
 		row[i] = v;
 		s2 = fmaf(v, v, s2);
+		sm2 += v;
 	}
 	if (!w_next)
 		return;
+	float mu2 = 0.0f;
+	if (ln) {
+		mu2 = block_sum(sm2, red) / (float)n;
+		s2 = 0.0f;
+		for (int i = threadIdx.x; i < n; i += SEQ_THREADS) {
+			const float d = row[i] - mu2;
+			s2 = fmaf(d, d, s2);
+		}
+	}
 	s2 = block_sum(s2, red);
 	const float r2 = 1.0f / sqrtf(s2 / (float)n + eps);
 	for (int i = threadIdx.x; i < n; i += SEQ_THREADS)
-		Hn[(size_t)t * n + i] = row[i] * r2 * w_next[i];
+		Hn[(size_t)t * n + i] = (row[i] - mu2) * r2 * w_next[i];
 }
 
 // ------------------------------------------------------------------ matrix products
-enum { EPI_NONE = 0, EPI_GLU_GELU = 1, EPI_GLU_CLAMP = 2, EPI_SIGMOID = 3 };
+enum { EPI_NONE = 0, EPI_GLU_GELU = 1, EPI_GLU_CLAMP = 2, EPI_SIGMOID = 3, EPI_GELU = 4 };
 
 // C[c_row(m)][n] = epi(sum_k A[a_row(m)][k] W[n][k]) for every batch z = blockIdx.z.
 struct GemmArgs {
@@ -288,6 +362,7 @@ __device__ __forceinline__ float epi_apply(const GemmArgs &a, float v, float v2,
 		return g * sq_sigmoid(1.702f * g) * (u + 1.0f);
 	}
 	case EPI_SIGMOID: return sq_sigmoid(v + b);
+	case EPI_GELU: return sq_gelu_tanh(v + b);
 	default: return v + b;
 	}
 }
@@ -1312,9 +1387,11 @@ static inline size_t att_lds_bytes(int rank) {
 	const int r4 = att_rank4(rank);
 	return sizeof(float) * ((size_t)ATT_BR * r4 + (size_t)ATT_KT * (r4 + 4) + ATT_BR * ATT_KT + 3 * ATT_BR);
 }
-// Ctx[r] = sum_s e^(m_s - M) acc_s / sum_s e^(m_s - M) l_s over the key splits of row r.
+// Ctx[r] = sum_s e^(m_s - M) acc_s / sum_s e^(m_s - M) l_s over the key splits of row r
+// (times gate[r] if given).
 __global__ __launch_bounds__(64) void seq_latent_merge_kernel(const float *__restrict__ part, int S, int rank,
-                                                              float *__restrict__ Ctx) {
+                                                              float *__restrict__ Ctx,
+                                                              const float *__restrict__ gate = nullptr) {
 	__shared__ float wsm[64]; // S <= 64: lane s holds split s
 	const int r = blockIdx.x, rank4 = att_rank4(rank), stride = rank4 + 4, lane = threadIdx.x;
 	const float *pp = part + (size_t)r * S * stride;
@@ -1322,7 +1399,7 @@ __global__ __launch_bounds__(64) void seq_latent_merge_kernel(const float *__res
 	const float l = lane < S ? pp[(size_t)lane * stride + rank4 + 1] : 0.0f;
 	const float M = wave_max(m);
 	const float w = expf(m - M);
-	const float inv = 1.0f / wave_sum(w * l);
+	const float inv = (gate ? gate[r] : 1.0f) / wave_sum(w * l);
 	wsm[lane] = w * inv;
 	__syncthreads();
 	for (int d = lane; d < rank; d += 64) {

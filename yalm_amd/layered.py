@@ -5,7 +5,8 @@ A layer-list design gives every layer its own token mixer and feed-forward
 description; a design registers a reader that turns its ``config.json`` into one and
 a packer that turns its checkpoint tensors into the engine's per-layer tensors
 (concatenated input projections, per-head transposed key up-projections, stacked
-experts). ``Sinulorn`` is the first such design.
+experts). ``Sinulorn`` (latent attention, recurrences, routed experts) and ``Lenuzen``
+(windowed / chunked softmax attention, plain feed-forwards) are such designs.
 
 Checkpoints are folders with ``config.json`` and ``model.safetensors`` (bf16
 matrices; read with yalmfile.read_yalm, the same container the .yalm files use).
@@ -21,8 +22,11 @@ import numpy as np
 
 from . import models as M
 
-MIX_LATENT, MIX_RGLRU, MIX_DELTA = 0, 1, 2
-FF_NONE, FF_DENSE, FF_MOE = 0, 1, 2
+MIX_LATENT, MIX_RGLRU, MIX_DELTA, MIX_ATTN = 0, 1, 2, 3
+FF_NONE, FF_DENSE, FF_MOE, FF_PLAIN = 0, 1, 2, 3
+NORM_RMS, NORM_LAYER = 0, 1
+MASK_CAUSAL, MASK_WINDOW, MASK_CHUNK = 0, 1, 2
+QK_NONE, QK_HEAD_UNIT, QK_WHOLE = 0, 1, 2
 
 
 @dataclasses.dataclass
@@ -49,6 +53,22 @@ class LayerSpec:
     limit: float = 0.0
     shared_ff: int = 0
     shared_limit: float = 0.0
+    # softmax attention over cached keys and values
+    mask_kind: int = MASK_CAUSAL
+    mask_size: int = 0
+    qk_norm: int = QK_NONE
+    v_norm: int = 0
+    sink: int = 0
+    out_gate: int = 0
+    rot_dims: int = 0
+    rot_orig: int = 0
+    rot_base: float = 10000.0
+    rot_factor: float = 0.0
+    rot_fast: float = 0.0
+    rot_slow: float = 0.0
+    in_biased: bool = False
+    head_temps: bool = False
+    talking: bool = False
 
     @property
     def in_rows(self) -> int:
@@ -57,6 +77,8 @@ class LayerSpec:
             return self.q_rank + (self.kv_rank if self.kv_from < 0 else 0)
         if self.mixer == MIX_RGLRU:
             return 2 * self.rec_width
+        if self.mixer == MIX_ATTN:
+            return self.heads * self.dim + self.kv_heads * (self.dim + self.vdim) + (self.heads if self.out_gate else 0)
         return 2 * self.kv_heads * self.dim + 2 * self.heads * self.vdim + 2 * self.heads
 
     @property
@@ -75,6 +97,11 @@ class LayeredConfig:
     norm_eps: float = 1e-5
     max_tokens: int = 4096
     weight_dtype: int = M.BF16
+    norm_kind: int = NORM_RMS
+    pre_norm: bool = True     # False: a sublayer reads the stream itself; only the closing norms exist
+    pos_embed: bool = True    # the sin / cos position vector added to the embedding
+    logit_scale: float = 1.0
+    tied_head: bool = False   # the logits read the embedding table
 
     def with_(self, **kw) -> "LayeredConfig":
         return dataclasses.replace(self, **kw)
@@ -84,9 +111,13 @@ def packed_shapes(c: LayeredConfig, l: LayerSpec) -> dict:
     """field -> (shape, kind) of one layer's engine tensors; kind "w": a matrix of the
     model's weight dtype, "f": f32."""
     W = c.width
-    out = {"norm1": ((W,), "f"), "norm1b": ((W,), "f")}
+    out = {"norm1b": ((W,), "f")}
+    if c.pre_norm:
+        out["norm1"] = ((W,), "f")
     if l.ff_kind != FF_NONE:
-        out.update(norm2=((W,), "f"), norm2b=((W,), "f"))
+        out["norm2b"] = ((W,), "f")
+        if c.pre_norm:
+            out["norm2"] = ((W,), "f")
     out["w_in"] = ((l.in_rows, W), "w")
     out["w_o"] = ((W, l.mix_out), "w")
     if l.mixer == MIX_LATENT:
@@ -103,10 +134,21 @@ def packed_shapes(c: LayeredConfig, l: LayerSpec) -> dict:
             gate_a=((l.blocks, bs, bs), "f"), gate_a_b=((l.rec_width,), "f"),
             gate_i=((l.blocks, bs, bs), "f"), gate_i_b=((l.rec_width,), "f"), lam=((l.rec_width,), "f"),
         )
+    elif l.mixer == MIX_ATTN:
+        if l.in_biased:
+            out["in_bias"] = ((l.in_rows,), "f")
+        if l.qk_norm == QK_WHOLE:
+            out.update(q_norm=((l.heads * l.dim,), "f"), kv_norm=((l.kv_heads * l.dim,), "f"))
+        if l.head_temps:
+            out["head_temp"] = ((l.heads,), "f")
+        if l.talking:
+            out["talk"] = ((l.heads, l.heads), "f")
     else:
         cc = 2 * l.kv_heads * l.dim + l.heads * l.vdim
         out.update(conv_w=((cc, l.conv), "f"), a_log=((l.heads,), "f"), dt_bias=((l.heads,), "f"),
                    out_norm=((l.vdim,), "f"))
+    if l.ff_kind == FF_PLAIN:
+        out.update(w_up=((l.ff, W), "w"), w_down=((W, l.ff), "w"))
     if l.ff_kind == FF_DENSE:
         out.update(w_gate=((l.ff, W), "w"), w_up=((l.ff, W), "w"), w_down=((W, l.ff), "w"))
     elif l.ff_kind == FF_MOE:
@@ -322,9 +364,147 @@ def sinulorn_random_tensors(cfg: dict, seed: int = 0, gain: float = 1.0) -> dict
     return out
 
 
+# ------------------------------------------------------------------ Lenuzen
+# Every layer: x += layer_norm(mixer(x)), then x += layer_norm(ff(x)); the sublayers read
+# the stream itself. Two mixers, both softmax attention over cached keys and values with
+# grouped key/value heads and partial interleaved rotary positions with rescaled frequencies:
+#   "attention":   biased projections, queries / keys / values divided by their per-head rms
+#                  (queries and keys after the rotation), a per-head score temperature, a
+#                  sliding window, a per-head sigmoid output gate;
+#   "attention_2": weighted rms norm of the whole query and key projections before the
+#                  rotation, scores mixed across heads by a [heads, heads] matrix, a chunked
+#                  mask, a softmax with a zero-score sink.
+# Feed-forward: w_down gelu(w_up x). Logits: the embedding table on the final norm, times
+# logit_scale.
+LENUZEN_MIXERS = ("attention", "attention_2")
+
+
+def lenuzen_config(cfg: dict, max_tokens: int = 4096, weight_dtype: int = M.BF16) -> LayeredConfig:
+    """config.json of a Lenuzen checkpoint -> LayeredConfig. Every size and every constant
+    that can differ between models of the design is read from cfg."""
+    layers = []
+    for e in cfg["layers"]:
+        m = e["mixer"]
+        if e["type"] not in LENUZEN_MIXERS:
+            raise ValueError(f"unknown mixer type {e['type']!r}")
+        rot = m["rot"]
+        sc = rot.get("scaling") or {}
+        s = LayerSpec(MIX_ATTN, heads=m["heads"], kv_heads=m.get("kv_heads", m["heads"]), dim=m["dim"], vdim=m["vdim"],
+                      attn_scale=float(m["scale"]), mask_size=int(m["mask"]["size"]), rot_dims=int(rot["dims"]),
+                      rot_base=float(rot["base"]), rot_factor=float(sc.get("factor", 0.0)),
+                      rot_orig=int(sc.get("original", 0)), rot_fast=float(sc.get("fast", 0.0)),
+                      rot_slow=float(sc.get("slow", 0.0)))
+        if e["type"] == "attention":
+            s.mask_kind, s.qk_norm, s.v_norm, s.out_gate = MASK_WINDOW, QK_HEAD_UNIT, 1, 1
+            s.in_biased = s.head_temps = True
+        else:
+            s.mask_kind, s.qk_norm, s.sink, s.talking = MASK_CHUNK, QK_WHOLE, 1, True
+        mlp = e.get("mlp")
+        if mlp:
+            if mlp["kind"] != "dense":
+                raise ValueError(f"unknown feed-forward kind {mlp['kind']!r}")
+            s.ff_kind, s.ff = FF_PLAIN, mlp["ff"]
+        layers.append(s)
+    return LayeredConfig(
+        arch="Lenuzen", width=cfg["width"], vocab=cfg["vocab"], layers=layers,
+        embed_scale=float(cfg["embedding"]["scale"]), norm_eps=float(cfg["norm"]["eps"]),
+        max_tokens=max_tokens, weight_dtype=weight_dtype, norm_kind=NORM_LAYER, pre_norm=False, pos_embed=False,
+        logit_scale=float(cfg.get("logit_scale", 1.0)), tied_head=True,
+    )
+
+
+def lenuzen_tensor_shapes(cfg: dict) -> dict:
+    """Checkpoint tensor name -> shape for a Lenuzen config.json."""
+    W = cfg["width"]
+    out = {"embed": (cfg["vocab"], W), "final.norm": (W,)}
+    for i, e in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", e["mixer"]
+        x = p + "mix."
+        H, G, D, V = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m["vdim"]
+        out[p + "norm1"] = (W,)
+        out[x + "q"], out[x + "k"], out[x + "v"], out[x + "o"] = (H * D, W), (G * D, W), (G * V, W), (W, H * V)
+        if e["type"] == "attention":
+            out[x + "q.b"], out[x + "k.b"], out[x + "v.b"] = (H * D,), (G * D,), (G * V,)
+            out[x + "temp"], out[x + "g"] = (H,), (H, W)
+        else:
+            out[x + "q.norm"], out[x + "k.norm"], out[x + "talk"] = (H * D,), (G * D,), (H, H)
+        if e.get("mlp"):
+            out[p + "norm2"] = (W,)
+            out[p + "mlp.up"], out[p + "mlp.down"] = (e["mlp"]["ff"], W), (W, e["mlp"]["ff"])
+    return out
+
+
+def lenuzen_pack(c: LayeredConfig, t: dict) -> dict:
+    """Checkpoint tensors -> the engine's tensors (see sinulorn_pack): q | k | v | gate rows
+    concatenated into w_in with one bias vector over all of them (zeros for the gate rows)."""
+    dt = c.weight_dtype
+
+    def w(*names):
+        parts = [_as_weight(t[n], dt) for n in names]
+        return parts[0] if len(parts) == 1 else np.ascontiguousarray(np.concatenate(parts, axis=0))
+
+    def f(name):
+        return np.ascontiguousarray(_as_f32(t[name]))
+
+    layers = []
+    for i, l in enumerate(c.layers):
+        p, x, m = f"l{i}.", f"l{i}.mix.", f"l{i}.mlp."
+        d = {"norm1b": f(p + "norm1")}
+        if l.out_gate:
+            d["w_in"] = w(x + "q", x + "k", x + "v", x + "g")
+        else:
+            d["w_in"] = w(x + "q", x + "k", x + "v")
+        if l.in_biased:
+            b = np.zeros(l.in_rows, np.float32)
+            nb = l.heads * l.dim + l.kv_heads * (l.dim + l.vdim)
+            b[:nb] = np.concatenate([f(x + "q.b"), f(x + "k.b"), f(x + "v.b")])
+            d["in_bias"] = b
+        if l.qk_norm == QK_WHOLE:
+            d.update(q_norm=f(x + "q.norm"), kv_norm=f(x + "k.norm"))
+        if l.head_temps:
+            d["head_temp"] = f(x + "temp")
+        if l.talking:
+            d["talk"] = f(x + "talk")
+        d["w_o"] = w(x + "o")
+        if l.ff_kind == FF_PLAIN:
+            d.update(norm2b=f(p + "norm2"), w_up=w(m + "up"), w_down=w(m + "down"))
+        want = packed_shapes(c, l)
+        if set(want) != set(d):
+            raise ValueError(f"layer {i}: packed tensors {sorted(d)} do not match the configuration's {sorted(want)}")
+        for k, (shape, _) in want.items():
+            if tuple(d[k].shape) != tuple(shape):
+                raise ValueError(f"layer {i}: tensor {k} has shape {d[k].shape}, the configuration gives {shape}")
+        layers.append(d)
+    emb = w("embed")
+    return {"embed": emb, "final_norm": f("final.norm"), "head": emb, "layers": layers}
+
+
+def lenuzen_random_tensors(cfg: dict, seed: int = 0, gain: float = 1.0) -> dict:
+    """Random checkpoint tensors for a Lenuzen config.json, as float32 arrays already rounded
+    to bf16 values (the f32 and bf16 engines and a float64 restatement see the same weights)."""
+    rng = np.random.default_rng(seed)
+    out = {}
+    for name, shape in lenuzen_tensor_shapes(cfg).items():
+        leaf = name.split(".")[-1]
+        if leaf in ("norm1", "norm2") or name.endswith(".norm"):
+            a = 1.0 + 0.2 * rng.standard_normal(shape)
+        elif leaf == "b":
+            a = 0.3 * rng.standard_normal(shape)
+        elif leaf == "temp":
+            a = rng.uniform(0.6, 1.6, shape)
+        elif leaf == "talk":
+            a = np.eye(shape[0]) + 0.25 * rng.standard_normal(shape)
+        elif leaf == "embed":
+            a = 0.1 * rng.standard_normal(shape)
+        else:
+            a = gain * rng.standard_normal(shape) / np.sqrt(shape[-1])
+        out[name] = bf16_to_f32(f32_to_bf16(a.astype(np.float32))).reshape(shape)
+    return out
+
+
 # ------------------------------------------------------------------ registry
 # design name (config.json "architecture") -> (config reader, weight packer)
-DESIGNS = {"Sinulorn": (sinulorn_config, sinulorn_pack)}
+DESIGNS = {"Sinulorn": (sinulorn_config, sinulorn_pack), "Lenuzen": (lenuzen_config, lenuzen_pack)}
 
 
 def read_checkpoint(path: str, max_tokens: int = 4096, weight_dtype: int = M.BF16):

@@ -142,7 +142,7 @@ class SeqLayer(ctypes.Structure):
     """yalm_seq_layer."""
 
     INTS = ("mixer", "heads", "kv_heads", "dim", "vdim", "kv_rank", "q_rank", "kv_from")
-    PTRS = ("norm1", "norm1b", "norm2", "norm2b", "q_norm", "kv_norm", "in_bias", "conv_w", "conv_b", "gate_a",
+    PTRS = ("norm1", "norm1b", "norm2", "norm2b", "q_norm", "kv_norm", "in_bias", "head_temp", "talk", "conv_w", "conv_b", "gate_a",
             "gate_a_b", "gate_i", "gate_i_b", "lam", "a_log", "dt_bias", "out_norm", "router", "shared_sg",
             "w_in", "w_uq", "w_ukt", "w_uv", "w_o", "w_gate", "w_up", "w_down", "ws_gate", "ws_up", "ws_down")
     _fields_ = (
@@ -150,13 +150,17 @@ class SeqLayer(ctypes.Structure):
                                       ("ff_kind", c_int), ("ff", c_int), ("experts", c_int), ("top", c_int),
                                       ("groups", c_int), ("groups_keep", c_int), ("router_scale", c_float),
                                       ("limit", c_float), ("shared_ff", c_int), ("shared_limit", c_float)]
+        + [(n, c_int) for n in ("mask_kind", "mask_size", "qk_norm", "v_norm", "sink", "out_gate", "rot_dims",
+                                "rot_orig")]
+        + [(n, c_float) for n in ("rot_base", "rot_factor", "rot_fast", "rot_slow")]
         + [(n, c_void_p) for n in PTRS]
     )
 
 
 class SeqConfig(ctypes.Structure):
     _fields_ = [("width", c_int), ("vocab", c_int), ("n_layers", c_int), ("max_tokens", c_int),
-                ("embed_scale", c_float), ("norm_eps", c_float), ("weight_dtype", c_int)]
+                ("embed_scale", c_float), ("norm_eps", c_float), ("weight_dtype", c_int), ("norm_kind", c_int),
+                ("pre_norm", c_int), ("pos_embed", c_int), ("logit_scale", c_float)]
 
 
 class SeqWeights(ctypes.Structure):
@@ -653,7 +657,8 @@ class SeqModel:
     def from_packed(cls, cfg, packed: dict) -> "SeqModel":
         self = cls(cfg)
         for k in ("embed", "final_norm", "head"):
-            self.ptrs[k] = self._up(packed[k])
+            # a tied head aliases the embedding table instead of a second upload
+            self.ptrs[k] = self.ptrs["embed"] if k == "head" and packed[k] is packed["embed"] else self._up(packed[k])
         for d in packed["layers"]:
             self.layer_ptrs.append({k: self._up(a) for k, a in d.items()})
         return self
@@ -685,7 +690,7 @@ class SeqModel:
             leaf = name.rsplit(".", 1)[-1]
             if kind == "w" or leaf in ("router", "gate_a", "gate_i", "shared_sg"):
                 scale, off = 1.7 / np.sqrt(fan_in or shape[-1]), 0.0
-            elif leaf.startswith("norm") or leaf in ("q_norm", "kv_norm", "out_norm", "final_norm"):
+            elif leaf.startswith("norm") or leaf in ("q_norm", "kv_norm", "out_norm", "final_norm", "head_temp"):
                 scale, off = 0.2, 1.0
             elif leaf == "conv_w":
                 scale, off = 0.5, 0.0
@@ -698,7 +703,7 @@ class SeqModel:
 
         self.ptrs["embed"] = make("embed", (cfg.vocab, cfg.width), "w", fan_in=100.0)
         self.ptrs["final_norm"] = make("final_norm", (cfg.width,), "f")
-        self.ptrs["head"] = make("head", (cfg.vocab, cfg.width), "w")
+        self.ptrs["head"] = self.ptrs["embed"] if cfg.tied_head else make("head", (cfg.vocab, cfg.width), "w")
         for i, l in enumerate(cfg.layers):
             self.layer_ptrs.append({k: make(f"l{i}.{k}", shape, kind)
                                     for k, (shape, kind) in layered.packed_shapes(cfg, l).items()})
@@ -715,7 +720,7 @@ class SeqModel:
                 else:
                     setattr(arr[i], name, getattr(l, name))
         sc = SeqConfig(cfg.width, cfg.vocab, len(cfg.layers), cfg.max_tokens, cfg.embed_scale, cfg.norm_eps,
-                       cfg.weight_dtype)
+                       cfg.weight_dtype, cfg.norm_kind, int(cfg.pre_norm), int(cfg.pos_embed), cfg.logit_scale)
         sw = SeqWeights(self.ptrs["embed"], self.ptrs["final_norm"], self.ptrs["head"], arr)
         return sc, sw, arr
 
