@@ -85,3 +85,86 @@ def test_restatement_router_respects_groups():
     s /= s.sum(1, keepdims=True)
     assert np.array_equal(idx[:, 0], s.argmax(1))
     assert np.allclose(wt[:, 0], 2.0 * s.max(1))
+
+
+# ------------------------------------------------------------------ Lenuzen
+def test_lenuzen_config_reads_every_size_and_constant():
+    import lenuzen_cases as LC
+
+    c = Ly.lenuzen_config(LC.MIXED, max_tokens=300)
+    assert (c.arch, c.width, c.vocab, c.embed_scale, c.norm_eps, c.max_tokens, c.logit_scale) == (
+        "Lenuzen", 96, 211, 5.0, 1e-5, 300, 0.75)
+    assert (c.norm_kind, c.pre_norm, c.pos_embed, c.tied_head) == (Ly.NORM_LAYER, False, False, True)
+    l0, l1, l2, l3, l4, l5 = c.layers
+    assert (l0.mixer, l0.heads, l0.kv_heads, l0.dim, l0.vdim, l0.mask_kind, l0.mask_size, l0.attn_scale) == (
+        Ly.MIX_ATTN, 3, 1, 32, 16, Ly.MASK_CHUNK, 7, 0.17)
+    assert (l0.qk_norm, l0.v_norm, l0.sink, l0.out_gate, l0.talking, l0.in_biased, l0.head_temps) == (
+        Ly.QK_WHOLE, 0, 1, 0, True, False, False)
+    assert (l0.rot_dims, l0.rot_base, l0.rot_factor, l0.rot_orig, l0.rot_fast, l0.rot_slow) == (32, 10000.0, 2.0, 64, 8.0, 2.0)
+    assert (l1.mask_kind, l1.mask_size, l1.qk_norm, l1.v_norm, l1.sink, l1.out_gate, l1.in_biased, l1.head_temps) == (
+        Ly.MASK_WINDOW, 9, Ly.QK_HEAD_UNIT, 1, 0, 1, True, True)
+    assert (l1.ff_kind, l1.ff, l2.ff_kind) == (Ly.FF_PLAIN, 40, Ly.FF_NONE)
+    assert l2.rot_factor == 0.0 and l3.rot_base == 500.0 and (l5.rot_factor, l5.rot_orig) == (8.0, 16)
+    assert l0.in_rows == 3 * 32 + 1 * (32 + 16) and l1.in_rows == 4 * 24 + 2 * (24 + 40) + 4
+    assert l1.mix_out == 4 * 40
+
+
+def test_lenuzen_unknown_names_are_refused():
+    import lenuzen_cases as LC
+
+    with pytest.raises(ValueError):
+        Ly.lenuzen_config(LC.config([("attention_3", LC.window(), None)]))
+    with pytest.raises(ValueError):
+        Ly.lenuzen_config(LC.config([("attention", LC.window(), {"kind": "moe", "ff": 8})]))
+
+
+def test_lenuzen_pack_concatenates_and_ties_the_head():
+    import lenuzen_cases as LC
+
+    cfg = LC.MIXED
+    t = Ly.lenuzen_random_tensors(cfg, seed=3)
+    assert set(t) == set(Ly.lenuzen_tensor_shapes(cfg))
+    for wdt in (M.F32, M.BF16):
+        c = Ly.lenuzen_config(cfg, weight_dtype=wdt)
+        p = Ly.lenuzen_pack(c, t)
+        f = (lambda a: a) if wdt == M.F32 else Ly.bf16_to_f32
+        assert p["head"] is p["embed"]
+        d1, l1 = p["layers"][1], c.layers[1]
+        assert np.array_equal(f(d1["w_in"]), np.concatenate([t["l1.mix." + n] for n in ("q", "k", "v", "g")]))
+        nb = l1.in_rows - l1.heads
+        assert np.array_equal(d1["in_bias"][:nb], np.concatenate([t["l1.mix." + n + ".b"] for n in ("q", "k", "v")]))
+        assert not d1["in_bias"][nb:].any()
+        assert np.array_equal(d1["head_temp"], t["l1.mix.temp"]) and np.array_equal(d1["norm1b"], t["l1.norm1"])
+        d0 = p["layers"][0]
+        assert np.array_equal(f(d0["w_in"]), np.concatenate([t["l0.mix." + n] for n in ("q", "k", "v")]))
+        assert np.array_equal(d0["talk"], t["l0.mix.talk"]) and np.array_equal(d0["q_norm"], t["l0.mix.q.norm"])
+        assert np.array_equal(f(d0["w_up"]), t["l0.mlp.up"]) and "norm2b" not in p["layers"][2]
+        for l, d in zip(c.layers, p["layers"]):
+            assert set(d) == set(Ly.packed_shapes(c, l))
+
+
+def test_lenuzen_restatement_is_causal_and_masks_hold():
+    """The restatement itself: logits at t do not depend on later tokens; a one-layer window
+    model's logits at t do not depend on tokens the window has left behind."""
+    import lenuzen_cases as LC
+    import lenuzen_ref as LR
+
+    cfg = LC.MIXED
+    w = {k: v.astype(np.float64) for k, v in Ly.lenuzen_random_tensors(cfg, seed=4).items()}
+    a = LC.tokens(cfg, 40, 1)
+    b = list(a)
+    b[30] = (b[30] + 1) % cfg["vocab"]
+    ra, rb = LR.forward(cfg, w, a), LR.forward(cfg, w, b)
+    assert np.array_equal(ra[:30], rb[:30]) and not np.allclose(ra[30], rb[30])
+    one = LC.ONLY_WINDOW
+    size = one["layers"][0]["mixer"]["mask"]["size"]
+    w1 = {k: v.astype(np.float64) for k, v in Ly.lenuzen_random_tensors(one, seed=5).items()}
+    a = LC.tokens(one, 30, 2)
+    b = list(a)
+    b[10] = (b[10] + 1) % one["vocab"]
+    ra, rb = LR.forward(one, w1, a), LR.forward(one, w1, b)
+    assert not np.allclose(ra[10 + size - 1], rb[10 + size - 1]) and np.allclose(ra[10 + size:], rb[10 + size:], atol=1e-12)
+    m = LR.visible("chunk", 4, 10)
+    assert m[5, 4] and not m[4, 3] and m[7, 4] and not m[8, 7] and not m[3, 4]
+    p = LR.softmax_rows(np.zeros((1, 3)), np.array([[True, True, False]]), True)
+    assert np.allclose(p, [[1 / 3, 1 / 3, 0.0]])
