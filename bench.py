@@ -79,6 +79,8 @@ def parse():
                          "(Sinulorn-shaped stacks, random bf16 weights) at a few real layer sizes, each beside a "
                          "Llama-shaped decoder of equal width, depth and feed-forward size; one JSON line")
     ap.add_argument("--layered-sizes", default="1024,2048,4096", help="model widths of the --layered legs")
+    ap.add_argument("--layered-design", default="sinulorn", choices=["sinulorn", "lenuzen"],
+                    help="which layer-list design the --layered stack is shaped like")
     return ap.parse_args()
 
 
@@ -531,6 +533,24 @@ def layered_stack(Ly, M, width, max_tokens):
                             weight_dtype=M.BF16)
 
 
+def lenuzen_stack(Ly, M, width, max_tokens):
+    """A Lenuzen-shaped stack at a real layer size: chunked attention with mixed scores and a
+    sink (two layers), then sliding-window attention with biases, temperatures and output
+    gates, twice over; head size 128, four query heads per key/value head, rotary positions
+    on half of a head, plain feed-forwards of 3.5 x width."""
+    heads = width // 128
+    kv = max(heads // 4, 1)
+    common = dict(heads=heads, kv_heads=kv, dim=128, vdim=128, attn_scale=128 ** -0.5, rot_dims=64, rot_base=50000.0,
+                  rot_factor=4.0, rot_orig=4096, rot_fast=32.0, rot_slow=1.0, ff_kind=Ly.FF_PLAIN, ff=width * 7 // 2)
+    chunked = dict(mask_kind=Ly.MASK_CHUNK, mask_size=2048, qk_norm=Ly.QK_WHOLE, sink=1, talking=True, **common)
+    windowed = dict(mask_kind=Ly.MASK_WINDOW, mask_size=1024, qk_norm=Ly.QK_HEAD_UNIT, v_norm=1, out_gate=1,
+                    in_biased=True, head_temps=True, **common)
+    layers = [Ly.LayerSpec(Ly.MIX_ATTN, **d) for d in (chunked, chunked, windowed, chunked, chunked, windowed)]
+    return Ly.LayeredConfig("Lenuzen", width, 32000, layers, embed_scale=1.0, norm_eps=1e-6, max_tokens=max_tokens,
+                            weight_dtype=M.BF16, norm_kind=Ly.NORM_LAYER, pre_norm=False, pos_embed=False,
+                            logit_scale=0.5, tied_head=True)
+
+
 def layered_bench(args, out_file):
     """--layered: tokens/s of a prompt portion (n = 2048 at position 0) and of single-token
     decoding (the device greedy loop at context ~1024) for the layer-list engine, and for a
@@ -544,7 +564,7 @@ def layered_bench(args, out_file):
     n_pf, ctx, steps = 2048, 1024, max(args.steps if args.steps != 256 else 64, 8)
     legs = []
     for width in [int(x) for x in args.layered_sizes.split(",")]:
-        cfg = layered_stack(Ly, M, width, n_pf + 64)
+        cfg = (lenuzen_stack if args.layered_design == "lenuzen" else layered_stack)(Ly, M, width, n_pf + 64)
         model = runtime.SeqModel.synthetic(cfg, seed=3)
         dec = runtime.SeqDecoder(model)
         pf_ms = dec.time_step(n_pf, 0, max(args.prefill_iters, 1))
@@ -580,8 +600,9 @@ def layered_bench(args, out_file):
             rd.close()
             dm.close()
         legs.append(leg)
-    print(json.dumps({"metric": "layer-list engine (Sinulorn-shaped stack, bf16) prefill and decode tok/s beside a "
-                                "Llama-shaped f16 decoder of equal width / depth / feed-forward size @1 GPU",
+    print(json.dumps({"metric": "layer-list engine (%s-shaped stack, bf16) prefill and decode tok/s beside a "
+                                "Llama-shaped f16 decoder of equal width / depth / feed-forward size @1 GPU"
+                                % args.layered_design.capitalize(),
                       "n_gpus": 1, "dtype": "bf16", "data": "synthetic", "legs": legs}), file=out_file, flush=True)
 
 

@@ -758,11 +758,11 @@ extern "C" int yalm_prefill_time(yalm_decoder d, int n, int iters, float *avg_ms
 }
 
 // The layer-list engine's door to the large-tile GEMM (seq.hip; device pointers, asynchronous
-// on st): C [M][ldc] f32 = A [M][lda] bf16 . W [N][K]^T bf16 (+ bias[n]). Same tiles, phases
+// on st): C [M][ldc] f32 = act(A [M][lda] bf16 . W [N][K]^T bf16 (+ bias[n])), act 1 = gelu. Same tiles, phases
 // and tile-width choice as the f16 prefill GEMMs; YALM_ERR_UNSUPPORTED (nothing launched)
 // when the shape does not fit them: K % 64, no tile width dividing N, rows not 16-byte aligned.
 int pf_gemm_bf16(const uint16_t *A, int lda, int M, int K, const uint16_t *W, int N, float *C, int ldc,
-                 const float *bias, hipStream_t st) {
+                 const float *bias, int act, hipStream_t st) {
 	static const PfForms f = pf_forms_default();
 	if (M <= 0 || K % pf::BK != 0 || lda % 8 != 0 || ((size_t)A | (size_t)W) % 16 != 0)
 		return YALM_ERR_UNSUPPORTED;
@@ -774,6 +774,7 @@ int pf_gemm_bf16(const uint16_t *A, int lda, int M, int K, const uint16_t *W, in
 	e.bias = bias;
 	e.ldc = ldc;
 	e.M = M;
+	e.act = act;
 	return launch_plain(f, bn, A, lda, M, K, K, one(W, N), N, e, st);
 }
 

@@ -113,7 +113,8 @@ struct E16StoreF32 {
 	}
 };
 
-// bf16 operands (epi_bf16), C[m][n] = acc (+ bias[n]) in f32: the layer-list engine's plain products
+// bf16 operands (epi_bf16), C[m][n] = act(acc (+ bias[n])) in f32: the layer-list engine's plain
+// products; act 1: the tanh form of gelu (an ungated feed-forward's first product)
 struct E16StoreF32B {
 	static constexpr bool NEEDS_LDS = false;
 	static constexpr bool BF16 = true;
@@ -121,6 +122,7 @@ struct E16StoreF32B {
 	float *c;
 	const float *bias;
 	int ldc, M;
+	int act = 0;
 	template <int FI, int FJ>
 	__device__ __forceinline__ void apply(f32x4_t (&acc)[FI][FJ], int m0, int n0, int lane, int, int) const {
 #pragma unroll
@@ -132,8 +134,11 @@ struct E16StoreF32B {
 #pragma unroll
 				for (int r = 0; r < 4; ++r) {
 					const int m = m0 + 16 * i + crow16(r, lane);
+					float v = acc[i][j][r] + b;
+					if (act == 1)
+						v = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
 					if (m < M)
-						c[(size_t)m * ldc + n] = acc[i][j][r] + b;
+						c[(size_t)m * ldc + n] = v;
 				}
 		}
 	}

@@ -25,7 +25,7 @@
 // library built from the shim and this unit alone has no prefill unit, and every product then
 // runs on this unit's general-shape kernels.
 int pf_gemm_bf16(const uint16_t *A, int lda, int M, int K, const uint16_t *W, int N, float *C, int ldc,
-                 const float *bias, hipStream_t st) __attribute__((weak));
+                 const float *bias, int act, hipStream_t st) __attribute__((weak));
 
 int pf_gemm_glu_bf16(const uint16_t *A, int lda, int M, int K, const uint16_t *Wg, const uint16_t *Wu, int hidden,
                      float *C, int ldc, int mode, float limit, hipStream_t st) __attribute__((weak));
@@ -278,7 +278,8 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 			bw = std::max(bw, (size_t)l.rec_width);
 			arena += (size_t)l.rec_width + (size_t)(l.conv - 1) * l.rec_width;
 		} else if (l.mixer == YALM_MIX_ATTN) {
-			bw = std::max({bw, (size_t)l.heads * l.dim, (size_t)l.heads * l.vdim});
+			// with score mixing a head's query spans the whole key row
+			bw = std::max({bw, (size_t)l.heads * l.dim * (l.talk ? l.kv_heads : 1), (size_t)l.heads * l.vdim});
 		} else {
 			const size_t cc = 2 * (size_t)l.kv_heads * l.dim + (size_t)l.heads * l.vdim;
 			bw = std::max({bw, cc, (size_t)l.heads * l.vdim, (size_t)2 * l.heads});
@@ -452,10 +453,14 @@ static int gemm(Seq *q, const GemmArgs &a, int batches = 1, int max_m = -1, bool
 		max_m = a.M;
 	if (f32w || q->c.weight_dtype == YALM_F32)
 		return gemm_t<WF32>(q, a, batches, max_m);
-	// plain products of long portions whose shape fits the large-tile GEMM of the prefill unit
+	// plain products of long portions whose shape fits the large-tile GEMM of the prefill unit;
+	// output columns past the last multiple of 128 (a few gate rows closing an input projection)
+	// run on the general kernel as a second, narrow product
 	const bool pair = a.W2 != nullptr && (a.epi == EPI_GLU_GELU || a.epi == EPI_GLU_CLAMP) && !a.bias;
+	const bool single = !a.W2 && (a.epi == EPI_NONE || a.epi == EPI_GELU);
+	const int n_big = pair ? (a.N % 64 == 0 ? a.N : 0) : (single ? a.N & ~127 : 0);
 	if (q->a16 && batches == 1 && max_m >= 2 * GB_BM && !a.rows && !a.w_sel && a.z_split == 0 && a.ldw == a.K &&
-	    a.K % 64 == 0 && (pair ? a.N % 64 == 0 : (!a.W2 && a.epi == EPI_NONE && a.N % 128 == 0))) {
+	    a.K % 64 == 0 && n_big > 0 && a.N - n_big <= 64) {
 		const size_t n8 = (size_t)a.M * (a.K / 8);
 		seq_to_bf16_kernel<<<(unsigned)std::min<size_t>((n8 + SEQ_THREADS - 1) / SEQ_THREADS, 4096), SEQ_THREADS, 0,
 		                     q->stream>>>(a.A, a.lda, a.M, a.K, q->a16);
@@ -463,7 +468,16 @@ static int gemm(Seq *q, const GemmArgs &a, int batches = 1, int max_m = -1, bool
 		const int rc =
 		    pair ? pf_gemm_glu_bf16(q->a16, a.K, a.M, a.K, (const uint16_t *)a.W, (const uint16_t *)a.W2, a.N, a.C, a.ldc,
 		                            a.epi == EPI_GLU_GELU ? 1 : 2, a.limit, q->stream)
-		         : pf_gemm_bf16(q->a16, a.K, a.M, a.K, (const uint16_t *)a.W, a.N, a.C, a.ldc, a.bias, q->stream);
+		         : pf_gemm_bf16(q->a16, a.K, a.M, a.K, (const uint16_t *)a.W, n_big, a.C, a.ldc, a.bias,
+		                        a.epi == EPI_GELU ? 1 : 0, q->stream);
+		if (rc == YALM_OK && n_big < a.N) {
+			GemmArgs t = a;
+			t.W = (const uint16_t *)a.W + (size_t)n_big * a.ldw;
+			t.C = a.C + n_big;
+			t.bias = a.bias ? a.bias + n_big : nullptr;
+			t.N = a.N - n_big;
+			return gemm_t<WBF16>(q, t, 1, max_m);
+		}
 		if (rc != YALM_ERR_UNSUPPORTED)
 			return rc;
 	}
@@ -632,16 +646,44 @@ static int mixer_delta(Seq *q, int li, int n) {
 	return gemm(q, plain(on, CV, l.w_o, CV, q->Y, c.width, n, c.width, CV));
 }
 
+template <int KS>
+static int attn_mfma_launch(Seq *q, int li, int n, const AttnArgs &a, const float *Q, int ldq, int qhs, const float *gate,
+                            float *ctx) {
+	const int rep = a.H / a.G, HW = rep >= 4 ? 4 : (rep >= 2 ? 2 : 1), NT = cdiv(a.V, 16);
+	const dim3 g(cdiv(n, 16 * (4 / HW)), a.G, cdiv(rep, HW));
+	const uint16_t *Kc = (const uint16_t *)q->cache[li], *Vc = (const uint16_t *)q->vcache[li];
+#define SAM_LAUNCH(N)                                                                                                  \
+	seq_attn_mfma_kernel<KS, N><<<g, SEQ_THREADS, 0, q->stream>>>(Q, ldq, qhs, Kc, Vc, a, n, HW, q->st, gate, ctx)
+	if (NT <= 2) SAM_LAUNCH(2);
+	else if (NT <= 4) SAM_LAUNCH(4);
+	else SAM_LAUNCH(8);
+#undef SAM_LAUNCH
+	HIPCHK(hipGetLastError());
+	return YALM_OK;
+}
+
 template <class CT>
 static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q, const float *gate, float *ctx) {
-	const yalm_seq_layer &l = q->L[li];
 	const bool talk = a.talk != nullptr;
-	const int Hb = talk ? a.H : a.H / a.G, V4n = (a.V + 3) / 4;
-	const int TQ = std::max(1, std::min(32 / Hb, n));
+	const int DK = talk ? a.G * a.D : a.D;
+	const int ldq = a.H * DK, qhs = DK;
+	if (sizeof(CT) == 2 && n > GEMV_MAX_M && DK <= 512 && a.V <= 128) { // portions over bf16 caches: the MFMA form
+		const int ks = cdiv(DK, 32);
+		if (ks <= 1) return attn_mfma_launch<1>(q, li, n, a, Q, ldq, qhs, gate, ctx);
+		if (ks <= 2) return attn_mfma_launch<2>(q, li, n, a, Q, ldq, qhs, gate, ctx);
+		if (ks <= 4) return attn_mfma_launch<4>(q, li, n, a, Q, ldq, qhs, gate, ctx);
+		if (ks <= 8) return attn_mfma_launch<8>(q, li, n, a, Q, ldq, qhs, gate, ctx);
+		return attn_mfma_launch<16>(q, li, n, a, Q, ldq, qhs, gate, ctx);
+	}
+	const int Hb = talk ? a.H : a.H / a.G, Gb = talk ? a.G : 1, V4n = (a.V + 3) / 4, D4 = (a.D + 3) & ~3;
+	// tokens per workgroup: up to 32 rows, their queries within 64 KB of LDS
+	int TQ = std::max(1, std::min(32 / Hb, n));
+	while (TQ > 1 && (size_t)TQ * Hb * Gb * D4 * sizeof(float) > 64 * 1024)
+		--TQ;
 	const int R = TQ * Hb;
 	const int S = n <= GEMV_MAX_M ? q->attn_splits[li] : 1;
 	const dim3 g(cdiv(n, TQ), S, talk ? 1 : a.G);
-	const size_t lds = sa_lds_bytes(R, a.H, a.D, a.V, talk);
+	const size_t lds = sa_lds_bytes(R, Gb, a.D, a.V);
 	const int na = cdiv(R * V4n, SEQ_THREADS);
 	const CT *Kc = (const CT *)q->cache[li], *Vc = (const CT *)q->vcache[li];
 #define SA_LAUNCH(NA)                                                                                                  \
@@ -652,8 +694,8 @@ static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q,
 			                           160 * 1024 - 64));                                                              \
 			attr_set = true;                                                                                           \
 		}                                                                                                              \
-		seq_attn_kernel<CT, NA><<<g, SEQ_THREADS, lds, q->stream>>>(Q, Kc, Vc, a, n, TQ, q->st, S == 1 ? gate : nullptr, \
-		                                                            ctx, q->att_part);                                 \
+		seq_attn_kernel<CT, NA><<<g, SEQ_THREADS, lds, q->stream>>>(Q, ldq, qhs, Kc, Vc, a, n, TQ, q->st,              \
+		                                                            S == 1 ? gate : nullptr, ctx, q->att_part);        \
 	} while (0)
 	if (na <= 1) SA_LAUNCH(1);
 	else if (na <= 2) SA_LAUNCH(2);
@@ -664,7 +706,6 @@ static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q,
 	if (S > 1)
 		seq_latent_merge_kernel<<<n * a.H, 64, 0, q->stream>>>(q->att_part, S, a.V, ctx, gate);
 	HIPCHK(hipGetLastError());
-	(void)l;
 	return YALM_OK;
 }
 
@@ -701,7 +742,7 @@ static int mixer_attn(Seq *q, int li, int n) {
 	a.temp = l.head_temp;
 	a.talk = l.talk;
 	a.eps = c.norm_eps;
-	const size_t rot_lds = (size_t)std::max(l.rot_dims, 2) * sizeof(float);
+	const size_t rot_lds = ((size_t)std::max(l.rot_dims, 2) + (l.talk ? (size_t)H * l.dim : 0)) * sizeof(float);
 	if (bf)
 		seq_attn_prep_kernel<uint16_t><<<n, SEQ_THREADS, rot_lds, q->stream>>>(q->Z, zin, a, q->st, Q, (uint16_t *)q->cache[li],
 		                                                                     (uint16_t *)q->vcache[li], gate);

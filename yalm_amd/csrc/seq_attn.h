@@ -5,6 +5,13 @@
 // window / chunked masks, a softmax with an optional zero-score sink, a per-head output gate.
 // Every option is a runtime argument, so another design can combine them differently.
 //
+// Scores mixed across heads, s'_h = sum_g talk[h][g] (q_g . k_kv(g)), are linear in the queries:
+// with q'_h = [sum_{g in c} talk[h][g] q_g for every key/value head c] (H D products per head,
+// once per token) they are s'_h = q'_h . (the whole key row of kv_heads x dim entries). The
+// projection kernel writes these mixed queries, and the attention kernels then see ordinary
+// independent heads whose keys are whole cache rows (DK = kv_heads x dim) while head h's
+// values stay those of its own key/value head.
+//
 // Positions and angles, the norms, scores, softmax weights and their weighted sums are f32
 // (the angle itself is evaluated in double: position * frequency loses bits in f32 at large
 // positions). The caches hold bf16 (WBF16 models) or f32 (WF32 models).
@@ -46,8 +53,9 @@ __device__ __forceinline__ void cache_store(CT *p, float v) {
 // ------------------------------------------------------------------ projections -> queries, cache rows, gates
 // One workgroup per token t at position p = st->pos + t, a wave per head. Z row: [q: H D | k: G D |
 // v: G V | gate: H] (biases already added). Queries leave scaled by scale * temp[h] in Q
-// [t][H D]; keys and values go to the cache rows p; gate[t][h] = sigmoid(z_gate[h]).
-// Dynamic LDS: rot_dims floats (cos | sin).
+// [t][H D], or, with score mixing, as the mixed queries Q [t][H][G D]; keys and values go to
+// the cache rows p; gate[t][h] = sigmoid(z_gate[h]).
+// Dynamic LDS: rot_dims floats (cos | sin) (+ H D floats with score mixing).
 template <class CT>
 __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_prep_kernel(const float *__restrict__ Z, int ldz, AttnArgs a,
                                                                     const StepState *__restrict__ st,
@@ -58,6 +66,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_prep_kernel(const float 
 	const int t = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
 	const int p = st->pos + t;
 	const int half = a.rot_dims >> 1;
+	float *qsh = rot + (a.rot_dims > 2 ? a.rot_dims : 2); // score mixing: the token's queries [H][D]
 	for (int i = tid; i < half; i += SEQ_THREADS) {
 		const double ang = (double)p * a.rot_freq[i];
 		rot[i] = (float)cos(ang) * a.rot_mag;
@@ -125,9 +134,12 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_prep_kernel(const float 
 			if (d >= n)
 				continue;
 			const float v = val[e] * mul;
-			if (kind == 0)
-				Q[(size_t)t * QN + hh * a.D + d] = v;
-			else if (kind == 1)
+			if (kind == 0) {
+				if (a.talk)
+					qsh[hh * a.D + d] = v;
+				else
+					Q[(size_t)t * QN + hh * a.D + d] = v;
+			} else if (kind == 1)
 				cache_store<CT>(Kc + (size_t)p * KN + hh * a.D + d, v);
 			else
 				cache_store<CT>(Vc + (size_t)p * VN + hh * a.V + d, v);
@@ -136,18 +148,31 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_prep_kernel(const float 
 	if (a.out_gate)
 		for (int h = tid; h < a.H; h += SEQ_THREADS)
 			gate[(size_t)t * a.H + h] = sq_sigmoid(z[QN + KN + VN + h]);
+	if (a.talk) {
+		__syncthreads();
+		const int rep = a.H / a.G, DK = a.G * a.D;
+		float *qo = Q + (size_t)t * a.H * DK;
+		for (int i = tid; i < a.H * DK; i += SEQ_THREADS) {
+			const int h = i / DK, c = (i % DK) / a.D, d = i % a.D;
+			float m = 0.0f;
+			for (int x = 0; x < rep; ++x)
+				m = fmaf(a.talk[h * a.H + c * rep + x], qsh[(c * rep + x) * a.D + d], m);
+			qo[i] = m;
+		}
+	}
 }
 
 // ------------------------------------------------------------------ attention, f32 FMA form
 // A workgroup owns TQ tokens x Hb heads (rows r = tq Hb + hl) and walks its share of the keys
-// they see in tiles of SA_KT. With score mixing (talk) a workgroup holds all heads of its
-// tokens (Hb = H, every key/value head in turn); without, the heads of one key/value head
-// (gridDim.z = G). Per tile: raw scores of every row (a lane per key), the mix across heads,
-// mask and running softmax per row, then the weighted sums of the value tile, each thread NA4
-// groups of 4 value entries of one row. Key splits (gridDim.y = S > 1; single tokens and short
-// portions): split s leaves (sums, running maximum, running sum) per row in `part` for
-// seq_latent_merge_kernel; the sink (a key of score 0 without a value) is split 0's starting
-// state. S == 1 writes the normalised, gated sums to Ctx [t][H V].
+// they see in tiles of SA_KT. Without score mixing the heads are those of one key/value head
+// (gridDim.z = G, key columns of that head); with it, all heads, whose (mixed) queries span
+// the whole key row, taken in G column chunks of D that accumulate into the same scores. Per
+// tile: scores of every row (a lane per key), mask and running softmax per row, then the
+// weighted sums of the value tile(s), each thread NA4 groups of 4 value entries of one row.
+// Key splits (gridDim.y = S > 1; single tokens and short portions): split s leaves (sums,
+// running maximum, running sum) per row in `part` for seq_latent_merge_kernel; the sink (a key
+// of score 0 without a value) is split 0's starting state. S == 1 writes the normalised,
+// gated sums to Ctx [t][H V].
 #define SA_KT 64
 #define SA_MAX_NA4 16
 
@@ -155,10 +180,10 @@ __host__ __device__ inline int sa_ldk(int D, int V) {
 	const int d4 = (D + 3) & ~3, v4 = (V + 3) & ~3;
 	return (d4 > v4 ? d4 : v4) + 4;
 }
-static inline size_t sa_lds_bytes(int R, int H, int D, int V, bool talk) {
+// R rows, Gb key column chunks per row
+static inline size_t sa_lds_bytes(int R, int Gb, int D, int V) {
 	const int d4 = (D + 3) & ~3;
-	return sizeof(float) * ((size_t)R * d4 + (size_t)SA_KT * sa_ldk(D, V) + (size_t)R * SA_KT * (talk ? 2 : 1) +
-	                        (talk ? (size_t)H * H : 0) + 5 * (size_t)R);
+	return sizeof(float) * ((size_t)R * Gb * d4 + (size_t)SA_KT * sa_ldk(D, V) + (size_t)R * SA_KT + 5 * (size_t)R);
 }
 
 // cs[jj][0 .. n4) = cache row kt + jj, columns col0 .. col0 + n (zeros past n and past k_end)
@@ -201,9 +226,11 @@ __device__ __forceinline__ void sa_fill_tile(float *cs, int ldk, const CT *cache
 	}
 }
 
+// Q: row (t, h) at Q + t ldq + h qhs, Gb chunks of D entries.
 template <class CT, int NA4>
-__global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__restrict__ Q, const CT *__restrict__ Kc,
-                                                               const CT *__restrict__ Vc, AttnArgs a, int n_tok, int TQ,
+__global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__restrict__ Q, int ldq, int qhs,
+                                                               const CT *__restrict__ Kc, const CT *__restrict__ Vc,
+                                                               AttnArgs a, int n_tok, int TQ,
                                                                const StepState *__restrict__ st,
                                                                const float *__restrict__ gate, float *__restrict__ Ctx,
                                                                float *__restrict__ part) {
@@ -213,13 +240,11 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 	const int Hb = talk ? H : rep, Gb = talk ? G : 1;
 	const int h0 = talk ? 0 : blockIdx.z * rep, g0 = talk ? 0 : blockIdx.z;
 	const int R = TQ * Hb;
-	const int D4 = (D + 3) & ~3, q4n = D4 >> 2, V4n = (V + 3) >> 2, ldk = sa_ldk(D, V);
-	float *qs = lds;                          // [R][D4]
-	float *cs = qs + R * D4;                  // [SA_KT][ldk]: the key tile, then the value tile
-	float *ps = cs + SA_KT * ldk;             // [R][SA_KT] raw scores, then softmax weights
-	float *ps2 = ps + R * SA_KT;              // talk: [R][SA_KT] mixed scores
-	float *tk = ps2 + (talk ? R * SA_KT : 0); // talk: [H][H]
-	float *mrun = tk + (talk ? H * H : 0);    // [R]
+	const int D4 = (D + 3) & ~3, q4n = D4 >> 2, V4n = (V + 3) >> 2, ldk = sa_ldk(D, V), ldqs = Gb * D4;
+	float *qs = lds;                  // [R][Gb][D4]
+	float *cs = qs + R * ldqs;        // [SA_KT][ldk]: a key chunk, then a value tile
+	float *ps = cs + SA_KT * ldk;     // [R][SA_KT] scores, then softmax weights
+	float *mrun = ps + R * SA_KT;     // [R]
 	float *lrun = mrun + R, *alpha = lrun + R;
 	int *rlo = (int *)(alpha + R), *rhi = rlo + R;
 	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -234,14 +259,11 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 		k_begin = klo + split * chunk;
 		k_end = min(khi + 1, k_begin + chunk);
 	}
-	for (int i = tid; i < R * D4; i += SEQ_THREADS) {
-		const int r = i / D4, d = i % D4;
+	for (int i = tid; i < R * ldqs; i += SEQ_THREADS) {
+		const int r = i / ldqs, c = (i % ldqs) / D4, d = i % D4;
 		const int t = t0 + r / Hb, h = h0 + r % Hb;
-		qs[i] = (t < n_tok && d < D) ? Q[((size_t)t * H + h) * D + d] : 0.0f;
+		qs[i] = (t < n_tok && d < D) ? Q[(size_t)t * ldq + (size_t)h * qhs + c * D + d] : 0.0f;
 	}
-	if (talk)
-		for (int i = tid; i < H * H; i += SEQ_THREADS)
-			tk[i] = a.talk[i];
 	const bool sink0 = a.sink && split == 0;
 	for (int r = tid; r < R; r += SEQ_THREADS) {
 		const int t = t0 + r / Hb;
@@ -255,61 +277,59 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 #pragma unroll
 	for (int x = 0; x < NA4; ++x)
 		acc[x] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
-	const int nrows_g = TQ * rep; // rows that read one key/value head
+	// few rows (single tokens): a row per wave and pass, so that every wave scores; else four
+	const int rg = R >= 4 * (SEQ_THREADS / 64) ? 4 : 1;
 	for (int kt = k_begin; kt < k_end; kt += SA_KT) {
-		// ---- raw scores
-		for (int gl = 0; gl < Gb; ++gl) {
+		// ---- scores
+		for (int c = 0; c < Gb; ++c) {
 			__syncthreads(); // the previous readers of cs are done
-			sa_fill_tile<CT>(cs, ldk, Kc, G * D, (g0 + gl) * D, D, kt, k_end);
+			sa_fill_tile<CT>(cs, ldk, Kc, G * D, (g0 + c) * D, D, kt, k_end);
 			__syncthreads();
 			const float4_t *cj = (const float4_t *)(cs + lane * ldk);
-			for (int i0 = wave * 4; i0 < nrows_g; i0 += 4 * (SEQ_THREADS / 64)) {
+			for (int i0 = wave * rg; i0 < R; i0 += rg * (SEQ_THREADS / 64)) {
 				int rr[4];
 #pragma unroll
-				for (int x = 0; x < 4; ++x) {
-					const int i = min(i0 + x, nrows_g - 1);
-					rr[x] = (i / rep) * Hb + gl * rep + (i % rep);
-				}
+				for (int x = 0; x < 4; ++x)
+					rr[x] = min(i0 + (x < rg ? x : 0), R - 1);
 				float s[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-				for (int d = 0; d < q4n; ++d) {
-					const float4_t c = cj[d];
+				if (rg == 4) {
+					for (int d = 0; d < q4n; ++d) {
+						const float4_t k4 = cj[d];
 #pragma unroll
-					for (int x = 0; x < 4; ++x) {
-						const float4_t qv = *(const float4_t *)(qs + rr[x] * D4 + 4 * d);
-						s[x] = fmaf(qv[0], c[0], s[x]);
-						s[x] = fmaf(qv[1], c[1], s[x]);
-						s[x] = fmaf(qv[2], c[2], s[x]);
-						s[x] = fmaf(qv[3], c[3], s[x]);
+						for (int x = 0; x < 4; ++x) {
+							const float4_t qv = *(const float4_t *)(qs + rr[x] * ldqs + c * D4 + 4 * d);
+							s[x] = fmaf(qv[0], k4[0], s[x]);
+							s[x] = fmaf(qv[1], k4[1], s[x]);
+							s[x] = fmaf(qv[2], k4[2], s[x]);
+							s[x] = fmaf(qv[3], k4[3], s[x]);
+						}
 					}
+				} else {
+					const float4_t *q0 = (const float4_t *)(qs + rr[0] * ldqs + c * D4);
+					float s1 = 0.0f, s2 = 0.0f, s3 = 0.0f;
+					for (int d = 0; d < q4n; ++d) {
+						const float4_t k4 = cj[d], qv = q0[d];
+						s[0] = fmaf(qv[0], k4[0], s[0]);
+						s1 = fmaf(qv[1], k4[1], s1);
+						s2 = fmaf(qv[2], k4[2], s2);
+						s3 = fmaf(qv[3], k4[3], s3);
+					}
+					s[0] = (s[0] + s1) + (s2 + s3);
 				}
 #pragma unroll
 				for (int x = 0; x < 4; ++x)
-					if (i0 + x < nrows_g)
-						ps[rr[x] * SA_KT + lane] = s[x];
+					if (x < rg && i0 + x < R) {
+						float *dst = ps + rr[x] * SA_KT + lane;
+						*dst = c == 0 ? s[x] : *dst + s[x];
+					}
 			}
 		}
 		__syncthreads();
-		// ---- mix across heads
-		const float *sc = ps;
-		if (talk) {
-			for (int pair = tid; pair < TQ * SA_KT; pair += SEQ_THREADS) {
-				const int tq = pair / SA_KT, key = pair % SA_KT;
-				const float *in = ps + (size_t)tq * H * SA_KT + key;
-				for (int h = 0; h < H; ++h) {
-					float m = 0.0f;
-					for (int g = 0; g < H; ++g)
-						m = fmaf(tk[h * H + g], in[g * SA_KT], m);
-					ps2[(tq * H + h) * SA_KT + key] = m;
-				}
-			}
-			__syncthreads();
-			sc = ps2;
-		}
 		// ---- mask and running softmax, a wave per row
 		for (int r = wave; r < R; r += SEQ_THREADS / 64) {
 			const int j = kt + lane;
 			const bool vis = j >= rlo[r] && j <= rhi[r] && j < k_end;
-			const float sv = vis ? sc[r * SA_KT + lane] : -FLT_MAX;
+			const float sv = vis ? ps[r * SA_KT + lane] : -FLT_MAX;
 			const float mold = mrun[r], lold = lrun[r];
 			const float mnew = fmaxf(mold, wave_max(sv));
 			const float p = vis ? expf(sv - mnew) : 0.0f;
@@ -347,11 +367,11 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 					const float4_t p = pr[j4];
 #pragma unroll
 					for (int e = 0; e < 4; ++e) {
-						const float4_t c = *(const float4_t *)(cs + (4 * j4 + e) * ldk + 4 * d4);
-						v[0] = fmaf(p[e], c[0], v[0]);
-						v[1] = fmaf(p[e], c[1], v[1]);
-						v[2] = fmaf(p[e], c[2], v[2]);
-						v[3] = fmaf(p[e], c[3], v[3]);
+						const float4_t c4 = *(const float4_t *)(cs + (4 * j4 + e) * ldk + 4 * d4);
+						v[0] = fmaf(p[e], c4[0], v[0]);
+						v[1] = fmaf(p[e], c4[1], v[1]);
+						v[2] = fmaf(p[e], c4[2], v[2]);
+						v[3] = fmaf(p[e], c4[3], v[3]);
 					}
 				}
 				acc[x] = v;
@@ -383,6 +403,183 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 				pp[4 * V4n] = mrun[r];
 				pp[4 * V4n + 1] = lrun[r];
 			}
+		}
+	}
+}
+
+// ------------------------------------------------------------------ attention, MFMA form (portions, bf16 cache)
+// v_mfma_f32_16x16x32_bf16 products with f32 accumulation; the f32 operands (queries, softmax
+// weights) enter as hi + lo bf16 pairs (hi = bf16(x), lo = bf16(x - hi): 16 significant bits),
+// the cached keys and values being bf16 already. Maximum, exponentials, running sums and the
+// rescaling of the sums stay f32, in the MFMA's C layout (row = 4 (lane >> 4) + reg, column =
+// lane & 15). A workgroup serves one key/value head g: its 4 waves are 4 / HW blocks of 16
+// tokens x HW query heads of g (blockIdx.z: which HW heads), so one key tile and one value tile
+// in LDS feed every wave. Keys in tiles of 32 from the first key the workgroup's first token
+// sees to its last token. KS = ceil(DK / 32), NT = ceil(V / 16).
+#define SAM_KT 32
+template <int KS, int NT>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_attn_mfma_kernel(const float *__restrict__ Q, int ldq, int qhs,
+                                                                    const uint16_t *__restrict__ Kc,
+                                                                    const uint16_t *__restrict__ Vc, AttnArgs a,
+                                                                    int n_tok, int HW, const StepState *__restrict__ st,
+                                                                    const float *__restrict__ gate,
+                                                                    float *__restrict__ Ctx) {
+	constexpr int DKP = 32 * KS, LDK = DKP + 8, LDT = SAM_KT + 8, LDP = SAM_KT + 8, VP = 16 * NT;
+	__shared__ __attribute__((aligned(16))) uint16_t Ks[SAM_KT * LDK];    // [key][key entry]
+	__shared__ __attribute__((aligned(16))) uint16_t VsT[VP * LDT];       // [value entry][key]
+	__shared__ __attribute__((aligned(16))) uint16_t Ps[4][2][16 * LDP];  // per wave: weights hi / lo [row][key]
+	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+	const int lr = lane & 15, lq = lane >> 4;
+	const int H = a.H, G = a.G, D = a.D, V = a.V, rep = H / G;
+	const bool talk = a.talk != nullptr;
+	const int DK = talk ? G * D : D, KL = G * D, VL = G * V;
+	const int g = blockIdx.y;
+	const int kcol = talk ? 0 : g * D;
+	const int TB = 4 / HW, tb = wave / HW, hl = blockIdx.z * HW + wave % HW;
+	const bool active = hl < rep;
+	const int h = g * rep + min(hl, rep - 1);
+	const int t0 = blockIdx.x * 16 * TB, tw0 = t0 + 16 * tb;
+	const int pos0 = st->pos;
+	const int t_last = min(t0 + 16 * TB, n_tok) - 1;
+	const int klo = attn_first_key(a.mask_kind, a.mask_size, pos0 + t0), khi = pos0 + t_last;
+	// the keys this wave's rows see: between the first row's first key and the last row's position
+	const int wlo = attn_first_key(a.mask_kind, a.mask_size, pos0 + min(tw0, n_tok - 1));
+	const int whi = pos0 + min(tw0 + 15, n_tok - 1);
+	const bool wave_on = active && tw0 < n_tok;
+	bf16x8_t qh[KS], ql[KS];
+	{
+		const int t = tw0 + lr;
+		const float *qrow = Q + (size_t)min(t, n_tok - 1) * ldq + (size_t)h * qhs;
+#pragma unroll
+		for (int sst = 0; sst < KS; ++sst) {
+			u32x4_t hi = {0, 0, 0, 0}, lo = {0, 0, 0, 0};
+#pragma unroll
+			for (int e = 0; e < 8; ++e) {
+				const int d = 32 * sst + 8 * lq + e;
+				const float x = (wave_on && t < n_tok && d < DK) ? qrow[d] : 0.0f;
+				const uint16_t hb = f2bf(x);
+				const uint16_t lb = f2bf(x - bf2f(hb));
+				hi[e >> 1] |= (uint32_t)hb << (16 * (e & 1));
+				lo[e >> 1] |= (uint32_t)lb << (16 * (e & 1));
+			}
+			qh[sst] = __builtin_bit_cast(bf16x8_t, hi);
+			ql[sst] = __builtin_bit_cast(bf16x8_t, lo);
+		}
+	}
+	int lo_[4], hi_[4];
+	float mrun[4], lrun[4];
+#pragma unroll
+	for (int r = 0; r < 4; ++r) {
+		const int t = tw0 + 4 * lq + r;
+		const bool ok = wave_on && t < n_tok;
+		lo_[r] = ok ? attn_first_key(a.mask_kind, a.mask_size, pos0 + t) : 0x7fffffff;
+		hi_[r] = ok ? pos0 + t : -1;
+		mrun[r] = a.sink ? 0.0f : -FLT_MAX;
+		lrun[r] = a.sink ? 1.0f : 0.0f;
+	}
+	f32x4a_t oacc[NT];
+#pragma unroll
+	for (int n = 0; n < NT; ++n)
+		oacc[n] = f32x4a_t{0.0f, 0.0f, 0.0f, 0.0f};
+	const bool kvec = DK % 8 == 0 && kcol % 8 == 0 && KL % 8 == 0 && (size_t)Kc % 16 == 0;
+	const bool vvec = V % 8 == 0 && VL % 8 == 0 && (size_t)Vc % 16 == 0;
+	for (int kt = klo; kt <= khi; kt += SAM_KT) {
+		__syncthreads(); // the previous tile's products have read Ks / VsT / Ps
+		for (int v = tid; v < SAM_KT * (DKP / 8); v += SEQ_THREADS) {
+			const int jj = v / (DKP / 8), d8 = (v % (DKP / 8)) * 8, j = kt + jj;
+			u32x4_t w = {0, 0, 0, 0};
+			if (j <= khi && d8 < DK) {
+				const uint16_t *src = Kc + (size_t)j * KL + kcol + d8;
+				if (kvec && d8 + 8 <= DK) {
+					w = load16(src);
+				} else {
+#pragma unroll
+					for (int e = 0; e < 8; ++e)
+						if (d8 + e < DK)
+							w[e >> 1] |= (uint32_t)src[e] << (16 * (e & 1));
+				}
+			}
+			*(u32x4_t *)(Ks + jj * LDK + d8) = w;
+		}
+		for (int v = tid; v < SAM_KT * (VP / 8); v += SEQ_THREADS) {
+			const int jj = v % SAM_KT, d8 = (v / SAM_KT) * 8, j = kt + jj;
+			u32x4_t w = {0, 0, 0, 0};
+			if (j <= khi && d8 < V) {
+				const uint16_t *src = Vc + (size_t)j * VL + g * V + d8;
+				if (vvec && d8 + 8 <= V) {
+					w = load16(src);
+				} else {
+#pragma unroll
+					for (int e = 0; e < 8; ++e)
+						if (d8 + e < V)
+							w[e >> 1] |= (uint32_t)src[e] << (16 * (e & 1));
+				}
+			}
+#pragma unroll
+			for (int e = 0; e < 8; ++e)
+				VsT[(d8 + e) * LDT + jj] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+		}
+		__syncthreads();
+		const bool need = wave_on && kt <= whi && kt + SAM_KT - 1 >= wlo;
+		if (need) {
+			f32x4a_t sacc[2] = {f32x4a_t{0.0f, 0.0f, 0.0f, 0.0f}, f32x4a_t{0.0f, 0.0f, 0.0f, 0.0f}};
+#pragma unroll
+			for (int jt = 0; jt < 2; ++jt)
+#pragma unroll
+				for (int sst = 0; sst < KS; ++sst) {
+					const bf16x8_t kb =
+					    __builtin_bit_cast(bf16x8_t, *(const u32x4_t *)(Ks + (16 * jt + lr) * LDK + 32 * sst + 8 * lq));
+					sacc[jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qh[sst], kb, sacc[jt], 0, 0, 0);
+					sacc[jt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ql[sst], kb, sacc[jt], 0, 0, 0);
+				}
+			float al[4];
+#pragma unroll
+			for (int r = 0; r < 4; ++r) {
+				const int j0 = kt + lr, j1 = kt + 16 + lr;
+				const bool v0 = j0 >= lo_[r] && j0 <= hi_[r], v1 = j1 >= lo_[r] && j1 <= hi_[r];
+				const float s0 = v0 ? sacc[0][r] : -FLT_MAX, s1 = v1 ? sacc[1][r] : -FLT_MAX;
+				const float mnew = fmaxf(mrun[r], row16_max(fmaxf(s0, s1)));
+				const float p0 = v0 ? expf(s0 - mnew) : 0.0f, p1 = v1 ? expf(s1 - mnew) : 0.0f;
+				al[r] = expf(mrun[r] - mnew);
+				lrun[r] = lrun[r] * al[r] + row16_sum(p0 + p1);
+				mrun[r] = mnew;
+				const int row = 4 * lq + r;
+				const uint16_t h0 = f2bf(p0), h1 = f2bf(p1);
+				Ps[wave][0][row * LDP + lr] = h0;
+				Ps[wave][0][row * LDP + 16 + lr] = h1;
+				Ps[wave][1][row * LDP + lr] = f2bf(p0 - bf2f(h0));
+				Ps[wave][1][row * LDP + 16 + lr] = f2bf(p1 - bf2f(h1));
+			}
+#pragma unroll
+			for (int n = 0; n < NT; ++n)
+#pragma unroll
+				for (int r = 0; r < 4; ++r)
+					oacc[n][r] *= al[r];
+		}
+		__syncthreads(); // the waves' weights are in LDS
+		if (need) {
+			const bf16x8_t ph = __builtin_bit_cast(bf16x8_t, *(const u32x4_t *)(&Ps[wave][0][lr * LDP + 8 * lq]));
+			const bf16x8_t pl = __builtin_bit_cast(bf16x8_t, *(const u32x4_t *)(&Ps[wave][1][lr * LDP + 8 * lq]));
+#pragma unroll
+			for (int n = 0; n < NT; ++n) {
+				const bf16x8_t vb = __builtin_bit_cast(bf16x8_t, *(const u32x4_t *)(VsT + (16 * n + lr) * LDT + 8 * lq));
+				oacc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ph, vb, oacc[n], 0, 0, 0);
+				oacc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pl, vb, oacc[n], 0, 0, 0);
+			}
+		}
+	}
+#pragma unroll
+	for (int r = 0; r < 4; ++r) {
+		const int t = tw0 + 4 * lq + r;
+		if (!wave_on || t >= n_tok)
+			continue;
+		const size_t row = (size_t)t * H + h;
+		const float f = (gate ? gate[row] : 1.0f) / lrun[r];
+#pragma unroll
+		for (int n = 0; n < NT; ++n) {
+			const int d = 16 * n + lr;
+			if (d < V)
+				Ctx[row * V + d] = oacc[n][r] * f;
 		}
 	}
 }
