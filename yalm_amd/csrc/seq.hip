@@ -278,7 +278,7 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 			bw = std::max(bw, (size_t)l.rec_width);
 			arena += (size_t)l.rec_width + (size_t)(l.conv - 1) * l.rec_width;
 		} else if (l.mixer == YALM_MIX_ATTN) {
-			// with score mixing a head's query spans the whole key row
+			// with score mixing a portion's queries span the whole key row
 			bw = std::max({bw, (size_t)l.heads * l.dim * (l.talk ? l.kv_heads : 1), (size_t)l.heads * l.vdim});
 		} else {
 			const size_t cc = 2 * (size_t)l.kv_heads * l.dim + (size_t)l.heads * l.vdim;
@@ -322,14 +322,14 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 			}
 		q->att_splits = std::max(1, std::min(32, cdiv(c.max_tokens, 2 * ATT_KT)));
 		size_t part = (size_t)(4 * ATT_BR + GEMV_MAX_M * max_h) * q->att_splits * (att_rank4(max_rank) + 4);
-		// attn: the keys a single token can see, split so that a workgroup walks about two tiles
+		// attn: the keys a single token can see, split so that a workgroup walks one tile (up to 64 splits)
 		q->attn_splits.assign(c.n_layers, 1);
 		for (int i = 0; i < c.n_layers; ++i) {
 			const yalm_seq_layer &l = q->L[i];
 			if (l.mixer != YALM_MIX_ATTN)
 				continue;
 			const int span = l.mask_kind == YALM_MASK_CAUSAL ? c.max_tokens : std::min(c.max_tokens, l.mask_size + GEMV_MAX_M);
-			q->attn_splits[i] = std::max(1, std::min(32, cdiv(span, 2 * SA_KT)));
+			q->attn_splits[i] = std::max(1, std::min(64, cdiv(span, SA_KT)));
 			part = std::max(part, (size_t)GEMV_MAX_M * l.heads * q->attn_splits[i] * (att_rank4(l.vdim) + 4));
 		}
 		STRY(sallocT(q, &q->att_part, part));
@@ -647,13 +647,12 @@ static int mixer_delta(Seq *q, int li, int n) {
 }
 
 template <int KS>
-static int attn_mfma_launch(Seq *q, int li, int n, const AttnArgs &a, const float *Q, int ldq, int qhs, const float *gate,
-                            float *ctx) {
+static int attn_mfma_launch(Seq *q, int li, int n, const AttnArgs &a, const float *Q, const float *gate, float *ctx) {
 	const int rep = a.H / a.G, HW = rep >= 4 ? 4 : (rep >= 2 ? 2 : 1), NT = cdiv(a.V, 16);
 	const dim3 g(cdiv(n, 16 * (4 / HW)), a.G, cdiv(rep, HW));
 	const uint16_t *Kc = (const uint16_t *)q->cache[li], *Vc = (const uint16_t *)q->vcache[li];
 #define SAM_LAUNCH(N)                                                                                                  \
-	seq_attn_mfma_kernel<KS, N><<<g, SEQ_THREADS, 0, q->stream>>>(Q, ldq, qhs, Kc, Vc, a, n, HW, q->st, gate, ctx)
+	seq_attn_mfma_kernel<KS, N><<<g, SEQ_THREADS, 0, q->stream>>>(Q, Kc, Vc, a, n, HW, q->st, gate, ctx)
 	if (NT <= 2) SAM_LAUNCH(2);
 	else if (NT <= 4) SAM_LAUNCH(4);
 	else SAM_LAUNCH(8);
@@ -666,16 +665,45 @@ template <class CT>
 static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q, const float *gate, float *ctx) {
 	const bool talk = a.talk != nullptr;
 	const int DK = talk ? a.G * a.D : a.D;
-	const int ldq = a.H * DK, qhs = DK;
 	if (sizeof(CT) == 2 && n > GEMV_MAX_M && DK <= 512 && a.V <= 128) { // portions over bf16 caches: the MFMA form
 		const int ks = cdiv(DK, 32);
-		if (ks <= 1) return attn_mfma_launch<1>(q, li, n, a, Q, ldq, qhs, gate, ctx);
-		if (ks <= 2) return attn_mfma_launch<2>(q, li, n, a, Q, ldq, qhs, gate, ctx);
-		if (ks <= 4) return attn_mfma_launch<4>(q, li, n, a, Q, ldq, qhs, gate, ctx);
-		if (ks <= 8) return attn_mfma_launch<8>(q, li, n, a, Q, ldq, qhs, gate, ctx);
-		return attn_mfma_launch<16>(q, li, n, a, Q, ldq, qhs, gate, ctx);
+		if (ks <= 1) return attn_mfma_launch<1>(q, li, n, a, Q, gate, ctx);
+		if (ks <= 2) return attn_mfma_launch<2>(q, li, n, a, Q, gate, ctx);
+		if (ks <= 4) return attn_mfma_launch<4>(q, li, n, a, Q, gate, ctx);
+		if (ks <= 8) return attn_mfma_launch<8>(q, li, n, a, Q, gate, ctx);
+		return attn_mfma_launch<16>(q, li, n, a, Q, gate, ctx);
 	}
 	const int Hb = talk ? a.H : a.H / a.G, Gb = talk ? a.G : 1, V4n = (a.V + 3) / 4, D4 = (a.D + 3) & ~3;
+	const CT *Kc = (const CT *)q->cache[li], *Vc = (const CT *)q->vcache[li];
+	const int rep = a.H / a.G;
+	const size_t dec_lds = sa_decode_lds_bytes(rep, DK, talk ? a.H * a.D : 0, a.H);
+	if (n == 1 && !a.q_mixed && dec_lds <= 96 * 1024) { // a decoded token: lanes read the cache rows themselves
+		const int S = q->attn_splits[li];
+		const dim3 g(S, a.G);
+		const size_t lds = dec_lds;
+		const int na = cdiv(rep * V4n, SEQ_THREADS);
+#define SD_LAUNCH(NA)                                                                                                  \
+	do {                                                                                                               \
+		static bool attr_set = false;                                                                                  \
+		if (!attr_set) {                                                                                               \
+			HIPCHK(hipFuncSetAttribute((const void *)seq_attn_decode_kernel<CT, NA>,                                    \
+			                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));                       \
+			attr_set = true;                                                                                           \
+		}                                                                                                              \
+		seq_attn_decode_kernel<CT, NA><<<g, SEQ_THREADS, lds, q->stream>>>(Q, Kc, Vc, a, q->st,                        \
+		                                                                   S == 1 ? gate : nullptr, ctx, q->att_part); \
+	} while (0)
+		if (na <= 1) SD_LAUNCH(1);
+		else if (na <= 2) SD_LAUNCH(2);
+		else if (na <= 4) SD_LAUNCH(4);
+		else if (na <= 8) SD_LAUNCH(8);
+		else SD_LAUNCH(16);
+#undef SD_LAUNCH
+		if (S > 1)
+			seq_latent_merge_kernel<<<a.H, 64, 0, q->stream>>>(q->att_part, S, a.V, ctx, gate);
+		HIPCHK(hipGetLastError());
+		return YALM_OK;
+	}
 	// tokens per workgroup: up to 32 rows, their queries within 64 KB of LDS
 	int TQ = std::max(1, std::min(32 / Hb, n));
 	while (TQ > 1 && (size_t)TQ * Hb * Gb * D4 * sizeof(float) > 64 * 1024)
@@ -685,7 +713,6 @@ static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q,
 	const dim3 g(cdiv(n, TQ), S, talk ? 1 : a.G);
 	const size_t lds = sa_lds_bytes(R, Gb, a.D, a.V);
 	const int na = cdiv(R * V4n, SEQ_THREADS);
-	const CT *Kc = (const CT *)q->cache[li], *Vc = (const CT *)q->vcache[li];
 #define SA_LAUNCH(NA)                                                                                                  \
 	do {                                                                                                               \
 		static bool attr_set = false; /* the kernel may use more dynamic LDS than the default limit */               \
@@ -694,7 +721,7 @@ static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q,
 			                           160 * 1024 - 64));                                                              \
 			attr_set = true;                                                                                           \
 		}                                                                                                              \
-		seq_attn_kernel<CT, NA><<<g, SEQ_THREADS, lds, q->stream>>>(Q, ldq, qhs, Kc, Vc, a, n, TQ, q->st,              \
+		seq_attn_kernel<CT, NA><<<g, SEQ_THREADS, lds, q->stream>>>(Q, Kc, Vc, a, n, TQ, q->st,                        \
 		                                                            S == 1 ? gate : nullptr, ctx, q->att_part);        \
 	} while (0)
 	if (na <= 1) SA_LAUNCH(1);
@@ -717,8 +744,9 @@ static int mixer_attn(Seq *q, int li, int n) {
 	const bool bf = c.weight_dtype == YALM_BF16;
 	const int zin = in_rows(l), H = l.heads, V = l.vdim;
 	float *Q = q->B[0], *gate = q->B[1], *ctx = q->B[2];
+	const int zmain = zin - (l.out_gate ? H : 0); // the gate rows are taken by the projection kernel itself
 	{
-		GemmArgs g = plain(q->In, c.width, l.w_in, c.width, q->Z, zin, n, zin, c.width);
+		GemmArgs g = plain(q->In, c.width, l.w_in, c.width, q->Z, zin, n, zmain, c.width);
 		g.bias = l.in_bias;
 		TRY(gemm(q, g));
 	}
@@ -742,13 +770,21 @@ static int mixer_attn(Seq *q, int li, int n) {
 	a.temp = l.head_temp;
 	a.talk = l.talk;
 	a.eps = c.norm_eps;
-	const size_t rot_lds = ((size_t)std::max(l.rot_dims, 2) + (l.talk ? (size_t)H * l.dim : 0)) * sizeof(float);
+	// portions: the projection kernel (one workgroup per token) mixes the queries itself
+	a.q_mixed = l.talk && n > GEMV_MAX_M ? 1 : 0;
+	const size_t rot_lds = ((size_t)std::max(l.rot_dims, 2) + (a.q_mixed ? (size_t)H * l.dim : 0)) * sizeof(float);
+	// a few tokens: their head jobs spread over several workgroups
+	const int jobs = H + 2 * l.kv_heads + (l.out_gate ? H : 0);
+	const dim3 pg(n, n <= GEMV_MAX_M ? cdiv(jobs, SEQ_THREADS / 64) : 1);
+	const float *gbias = l.in_bias ? l.in_bias + zmain : nullptr;
 	if (bf)
-		seq_attn_prep_kernel<uint16_t><<<n, SEQ_THREADS, rot_lds, q->stream>>>(q->Z, zin, a, q->st, Q, (uint16_t *)q->cache[li],
-		                                                                     (uint16_t *)q->vcache[li], gate);
+		seq_attn_prep_kernel<uint16_t><<<pg, SEQ_THREADS, rot_lds, q->stream>>>(
+		    q->Z, zin, a, q->st, Q, (uint16_t *)q->cache[li], (uint16_t *)q->vcache[li], gate, q->In, c.width,
+		    (const uint16_t *)l.w_in + (size_t)zmain * c.width, gbias);
 	else
-		seq_attn_prep_kernel<float><<<n, SEQ_THREADS, rot_lds, q->stream>>>(q->Z, zin, a, q->st, Q, (float *)q->cache[li],
-		                                                                  (float *)q->vcache[li], gate);
+		seq_attn_prep_kernel<float><<<pg, SEQ_THREADS, rot_lds, q->stream>>>(
+		    q->Z, zin, a, q->st, Q, (float *)q->cache[li], (float *)q->vcache[li], gate, q->In, c.width,
+		    (const float *)l.w_in + (size_t)zmain * c.width, gbias);
 	HIPCHK(hipGetLastError());
 	const float *gp = l.out_gate ? gate : nullptr;
 	TRY(bf ? attn_core_t<uint16_t>(q, li, n, a, Q, gp, ctx) : attn_core_t<float>(q, li, n, a, Q, gp, ctx));

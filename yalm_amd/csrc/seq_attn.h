@@ -8,13 +8,15 @@
 // Scores mixed across heads, s'_h = sum_g talk[h][g] (q_g . k_kv(g)), are linear in the queries:
 // with q'_h = [sum_{g in c} talk[h][g] q_g for every key/value head c] (H D products per head,
 // once per token) they are s'_h = q'_h . (the whole key row of kv_heads x dim entries). The
-// projection kernel writes these mixed queries, and the attention kernels then see ordinary
-// independent heads whose keys are whole cache rows (DK = kv_heads x dim) while head h's
-// values stay those of its own key/value head.
+// mixed queries are built once per token (by the projection kernel for portions, by the
+// attention kernel as it loads the queries for a few tokens, whose projection is spread over
+// several workgroups), and the attention kernels then see ordinary independent heads whose
+// keys are whole cache rows (DK = kv_heads x dim) while head h's values stay those of its own
+// key/value head.
 //
 // Positions and angles, the norms, scores, softmax weights and their weighted sums are f32
-// (the angle itself is evaluated in double: position * frequency loses bits in f32 at large
-// positions). The caches hold bf16 (WBF16 models) or f32 (WF32 models).
+// (the angle itself is evaluated and reduced to [-pi, pi] in double: position * frequency
+// loses bits in f32 at large positions). The caches hold bf16 (WBF16 models) or f32 (WF32 models).
 #pragma once
 
 #include "seq_kernels.h"
@@ -31,6 +33,7 @@ struct AttnArgs {
 	const float *temp;        // [H] or null
 	const float *talk;        // [H][H] or null
 	float eps;
+	int q_mixed;              // talk: the projection kernel has already written the mixed queries [t][H][G D]
 };
 
 // First key position that position p sees.
@@ -42,6 +45,24 @@ __host__ __device__ __forceinline__ int attn_first_key(int mask_kind, int mask_s
 	return 0;
 }
 
+// Entry d of head h's query as the attention kernels use it: the query itself, or with score
+// mixing (talk != null) entry d of the mixed query over the whole key row. Q: the projection
+// kernel's output, [t][H][D] queries or (mixed) [t][H][G D] mixed queries.
+__device__ __forceinline__ float attn_query(const float *__restrict__ Q, int t, const float *__restrict__ talk,
+                                            bool mixed, int H, int G, int D, int h, int d) {
+	if (!talk)
+		return Q[((size_t)t * H + h) * D + d];
+	if (mixed)
+		return Q[((size_t)t * H + h) * G * D + d];
+	const float *qt = Q + (size_t)t * H * D;
+	const int rep = H / G;
+	const int c = d / D, dd = d - c * D;
+	float m = 0.0f;
+	for (int x = 0; x < rep; ++x)
+		m = fmaf(talk[h * H + c * rep + x], qt[(c * rep + x) * D + dd], m);
+	return m;
+}
+
 template <class CT>
 __device__ __forceinline__ void cache_store(CT *p, float v) {
 	if constexpr (sizeof(CT) == 2)
@@ -51,26 +72,37 @@ __device__ __forceinline__ void cache_store(CT *p, float v) {
 }
 
 // ------------------------------------------------------------------ projections -> queries, cache rows, gates
-// One workgroup per token t at position p = st->pos + t, a wave per head. Z row: [q: H D | k: G D |
-// v: G V | gate: H] (biases already added). Queries leave scaled by scale * temp[h] in Q
-// [t][H D], or, with score mixing, as the mixed queries Q [t][H][G D]; keys and values go to
-// the cache rows p; gate[t][h] = sigmoid(z_gate[h]).
-// Dynamic LDS: rot_dims floats (cos | sin) (+ H D floats with score mixing).
+// Token t (blockIdx.x) at position p = st->pos + t; a wave per head job: the H query heads, G
+// key heads, G value heads and, with an output gate, H gate heads; the workgroups of a token
+// (gridDim.y) take the jobs in turn, so a single decoded token spreads over several workgroups
+// while a long portion runs one workgroup per token. Z row: [q: H D | k: G D | v: G V] (biases
+// already added). Queries leave scaled by scale * temp[h] in Q [t][H D], or (a.q_mixed, one
+// workgroup per token) as the mixed queries [t][H][G D]; keys and values go to the cache rows p. A gate job is a short dot product taken here, from the sublayer's input
+// row X[t] and the gate rows Wg [H][width] (stored as CT, the model's matrix type): gate[t][h]
+// = sigmoid(Wg[h] . X[t] + gate_bias[h]). Dynamic LDS: rot_dims floats (cos | sin) (+ H D
+// floats with a.q_mixed).
 template <class CT>
 __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_prep_kernel(const float *__restrict__ Z, int ldz, AttnArgs a,
                                                                     const StepState *__restrict__ st,
                                                                     float *__restrict__ Q, CT *__restrict__ Kc,
-                                                                    CT *__restrict__ Vc, float *__restrict__ gate) {
+                                                                    CT *__restrict__ Vc, float *__restrict__ gate,
+                                                                    const float *__restrict__ X, int width,
+                                                                    const CT *__restrict__ Wg,
+                                                                    const float *__restrict__ gate_bias) {
 	extern __shared__ float rot[];
 	__shared__ float red[SEQ_THREADS / 64];
+	constexpr int NW = SEQ_THREADS / 64;
 	const int t = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
 	const int p = st->pos + t;
 	const int half = a.rot_dims >> 1;
-	float *qsh = rot + (a.rot_dims > 2 ? a.rot_dims : 2); // score mixing: the token's queries [H][D]
+	float *qsh = rot + (a.rot_dims > 2 ? a.rot_dims : 2); // a.q_mixed: the token's queries [H][D]
 	for (int i = tid; i < half; i += SEQ_THREADS) {
+		// position x frequency and its reduction to [-pi, pi] in double, cos / sin of that in f32
+		const double two_pi = 6.283185307179586476925286766559;
 		const double ang = (double)p * a.rot_freq[i];
-		rot[i] = (float)cos(ang) * a.rot_mag;
-		rot[half + i] = (float)sin(ang) * a.rot_mag;
+		const float red_ang = (float)(ang - two_pi * rint(ang * (1.0 / two_pi)));
+		rot[i] = cosf(red_ang) * a.rot_mag;
+		rot[half + i] = sinf(red_ang) * a.rot_mag;
 	}
 	const float *z = Z + (size_t)t * ldz;
 	const int QN = a.H * a.D, KN = a.G * a.D, VN = a.G * a.V;
@@ -87,8 +119,45 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_prep_kernel(const float 
 		rk = 1.0f / sqrtf(block_sum(s, red) / (float)KN + a.eps);
 	}
 	__syncthreads();
-	const int jobs = a.H + 2 * a.G;
-	for (int job = wave; job < jobs; job += SEQ_THREADS / 64) {
+	const int jobs = a.H + 2 * a.G + (a.out_gate ? a.H : 0);
+	for (int job = blockIdx.y * NW + wave; job < jobs; job += gridDim.y * NW) {
+		if (job >= a.H + 2 * a.G) { // an output gate
+			constexpr int EPL = sizeof(CT) == 2 ? 8 : 4;
+			const int h = job - a.H - 2 * a.G;
+			const float *x = X + (size_t)t * width;
+			const CT *wr = Wg + (size_t)h * width;
+			float s = 0.0f;
+			if (width % EPL == 0 && (size_t)Wg % 16 == 0 && (size_t)X % 16 == 0) {
+				for (int k = lane * EPL; k < width; k += 64 * EPL) {
+					float wf[EPL];
+					if constexpr (sizeof(CT) == 2)
+						WBF16::unpack(load16(wr + k), wf);
+					else
+						WF32::unpack(load16(wr + k), wf);
+#pragma unroll
+					for (int e = 0; e < EPL; e += 4) {
+						const float4_t xv = *(const float4_t *)(x + k + e);
+						s = fmaf(wf[e], xv[0], s);
+						s = fmaf(wf[e + 1], xv[1], s);
+						s = fmaf(wf[e + 2], xv[2], s);
+						s = fmaf(wf[e + 3], xv[3], s);
+					}
+				}
+			} else {
+				for (int k = lane; k < width; k += 64) {
+					float wv;
+					if constexpr (sizeof(CT) == 2)
+						wv = bf2f(wr[k]);
+					else
+						wv = wr[k];
+					s = fmaf(wv, x[k], s);
+				}
+			}
+			s = wave_sum(s);
+			if (lane == 0)
+				gate[(size_t)t * a.H + h] = sq_sigmoid(s + (gate_bias ? gate_bias[h] : 0.0f));
+			continue;
+		}
 		const int kind = job < a.H ? 0 : (job < a.H + a.G ? 1 : 2); // query, key, value head
 		const int hh = kind == 0 ? job : (kind == 1 ? job - a.H : job - a.H - a.G);
 		const int n = kind == 2 ? a.V : a.D;
@@ -111,8 +180,8 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_prep_kernel(const float 
 						u = u * rw * nw[d0];
 						w = w * rw * nw[d1];
 					}
-					const float c = rot[d >> 1], s = rot[half + (d >> 1)];
-					v = (d & 1) ? w * c + u * s : u * c - w * s;
+					const float c = rot[d >> 1], sn = rot[half + (d >> 1)];
+					v = (d & 1) ? w * c + u * sn : u * c - w * sn;
 				} else {
 					v = src[d];
 					if (nw)
@@ -135,7 +204,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_prep_kernel(const float 
 				continue;
 			const float v = val[e] * mul;
 			if (kind == 0) {
-				if (a.talk)
+				if (a.q_mixed)
 					qsh[hh * a.D + d] = v;
 				else
 					Q[(size_t)t * QN + hh * a.D + d] = v;
@@ -145,19 +214,20 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_prep_kernel(const float 
 				cache_store<CT>(Vc + (size_t)p * VN + hh * a.V + d, v);
 		}
 	}
-	if (a.out_gate)
-		for (int h = tid; h < a.H; h += SEQ_THREADS)
-			gate[(size_t)t * a.H + h] = sq_sigmoid(z[QN + KN + VN + h]);
-	if (a.talk) {
+	if (a.q_mixed) { // q'[h][c D + d] = sum_x talk[h][c rep + x] q[c rep + x][d]
 		__syncthreads();
 		const int rep = a.H / a.G, DK = a.G * a.D;
 		float *qo = Q + (size_t)t * a.H * DK;
-		for (int i = tid; i < a.H * DK; i += SEQ_THREADS) {
-			const int h = i / DK, c = (i % DK) / a.D, d = i % a.D;
-			float m = 0.0f;
-			for (int x = 0; x < rep; ++x)
-				m = fmaf(a.talk[h * a.H + c * rep + x], qsh[(c * rep + x) * a.D + d], m);
-			qo[i] = m;
+		for (int cd = tid; cd < DK; cd += SEQ_THREADS) {
+			const int c = cd / a.D, d = cd - c * a.D;
+			const float *qc = qsh + c * rep * a.D + d;
+			for (int h = 0; h < a.H; ++h) {
+				const float *tr = a.talk + h * a.H + c * rep;
+				float m = 0.0f;
+				for (int x = 0; x < rep; ++x)
+					m = fmaf(tr[x], qc[x * a.D], m);
+				qo[(size_t)h * DK + cd] = m;
+			}
 		}
 	}
 }
@@ -226,9 +296,9 @@ __device__ __forceinline__ void sa_fill_tile(float *cs, int ldk, const CT *cache
 	}
 }
 
-// Q: row (t, h) at Q + t ldq + h qhs, Gb chunks of D entries.
+// Q [t][H D]: the projection kernel's queries.
 template <class CT, int NA4>
-__global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__restrict__ Q, int ldq, int qhs,
+__global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__restrict__ Q,
                                                                const CT *__restrict__ Kc, const CT *__restrict__ Vc,
                                                                AttnArgs a, int n_tok, int TQ,
                                                                const StepState *__restrict__ st,
@@ -262,7 +332,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 	for (int i = tid; i < R * ldqs; i += SEQ_THREADS) {
 		const int r = i / ldqs, c = (i % ldqs) / D4, d = i % D4;
 		const int t = t0 + r / Hb, h = h0 + r % Hb;
-		qs[i] = (t < n_tok && d < D) ? Q[(size_t)t * ldq + (size_t)h * qhs + c * D + d] : 0.0f;
+		qs[i] = (t < n_tok && d < D) ? attn_query(Q, t, a.talk, a.q_mixed != 0, H, G, D, h, c * D + d) : 0.0f;
 	}
 	const bool sink0 = a.sink && split == 0;
 	for (int r = tid; r < R; r += SEQ_THREADS) {
@@ -407,6 +477,258 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 	}
 }
 
+// ------------------------------------------------------------------ attention, single token
+// One decoded token: nothing is staged through LDS but the queries. A workgroup owns one key
+// split (gridDim.x = S) of the heads of one key/value head (gridDim.y = G; with score mixing
+// their mixed queries meet the whole key row); a lane owns a key and reads its cache row itself, 16 bytes at a time,
+// eight loads in flight; wave w takes a quarter of the key entries against every head's
+// queries (LDS broadcasts) and leaves partial scores in LDS; wave w then adds them up and
+// normalises heads w, w + 4, ...; then every thread sums NA4 groups of 4 value entries of one
+// head straight from the value rows. Partial results per split as in
+// seq_attn_kernel (S == 1 writes Ctx).
+template <class CT, int NA4>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_attn_decode_kernel(const float *__restrict__ Q,
+                                                                      const CT *__restrict__ Kc,
+                                                                      const CT *__restrict__ Vc, AttnArgs a,
+                                                                      const StepState *__restrict__ st,
+                                                                      const float *__restrict__ gate,
+                                                                      float *__restrict__ Ctx, float *__restrict__ part) {
+	extern __shared__ __attribute__((aligned(16))) float lds[];
+	constexpr int NW = SEQ_THREADS / 64;
+	constexpr int EPL = sizeof(CT) == 2 ? 8 : 4; // cache entries per 16-byte load
+	constexpr int HP = 16;                        // heads per pass over a key slice
+	const int H = a.H, G = a.G, D = a.D, V = a.V, rep = H / G;
+	const bool talk = a.talk != nullptr;
+	const int Hb = rep, h0 = blockIdx.y * rep; // the heads of one key/value head
+	const int DK = talk ? G * D : D, KL = G * D, VL = G * V, kcol = talk ? 0 : blockIdx.y * D;
+	const int DK8 = (DK + 7) & ~7, V4n = (V + 3) >> 2;
+	float *qs = lds;               // [Hb][DK8]
+	float *ps = qs + Hb * DK8;     // [Hb][SA_KT] softmax weights
+	float *pw = ps + Hb * SA_KT;   // [NW][Hb][SA_KT] the waves' partial scores
+	float *mrun = pw + NW * Hb * SA_KT; // [Hb]
+	float *lrun = mrun + Hb, *alpha = lrun + Hb;
+	const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+	const int S = gridDim.x, split = blockIdx.x;
+	const int pos = st->pos;
+	const int klo = attn_first_key(a.mask_kind, a.mask_size, pos);
+	int k_begin = klo, k_end = pos + 1;
+	if (S > 1) {
+		const int nkeys = pos - klo + 1;
+		const int chunk = (((nkeys + S - 1) / S) + SA_KT - 1) & ~(SA_KT - 1);
+		k_begin = klo + split * chunk;
+		k_end = min(pos + 1, k_begin + chunk);
+	}
+	if (talk && !a.q_mixed) { // the token's queries and the mixing matrix through LDS, then the mixed queries
+		float *qraw = alpha + Hb, *tk = qraw + H * D;
+		for (int i = tid; i < H * D; i += SEQ_THREADS)
+			qraw[i] = Q[i];
+		for (int i = tid; i < H * H; i += SEQ_THREADS)
+			tk[i] = a.talk[i];
+		__syncthreads();
+		for (int cd = tid; cd < DK8; cd += SEQ_THREADS) {
+			const int c = cd / D, d = cd - c * D;
+			for (int hl = 0; hl < Hb; ++hl) {
+				float m = 0.0f;
+				if (cd < DK)
+					for (int x = 0; x < rep; ++x)
+						m = fmaf(tk[(h0 + hl) * H + c * rep + x], qraw[(c * rep + x) * D + d], m);
+				qs[hl * DK8 + cd] = m;
+			}
+		}
+	} else {
+		for (int i = tid; i < Hb * DK8; i += SEQ_THREADS) {
+			const int hl = i / DK8, d = i % DK8;
+			qs[i] = d < DK ? attn_query(Q, 0, a.talk, a.q_mixed != 0, H, G, D, h0 + hl, d) : 0.0f;
+		}
+	}
+	const bool sink0 = a.sink && split == 0;
+	for (int r = tid; r < Hb; r += SEQ_THREADS) {
+		mrun[r] = sink0 ? 0.0f : -FLT_MAX;
+		lrun[r] = sink0 ? 1.0f : 0.0f;
+		alpha[r] = 1.0f;
+	}
+	float4_t acc[NA4];
+#pragma unroll
+	for (int x = 0; x < NA4; ++x)
+		acc[x] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+	const bool kvec = DK % EPL == 0 && kcol % EPL == 0 && KL % EPL == 0 && (size_t)Kc % 16 == 0;
+	const bool vvec = V % 4 == 0 && VL % 4 == 0 && (size_t)Vc % 16 == 0;
+	const int DKw = (((DK + NW - 1) / NW) + EPL - 1) / EPL * EPL; // key entries per wave
+	const int dlo = min(wave * DKw, DK), dhi = min(DK, dlo + DKw);
+	__syncthreads();
+	for (int kt = k_begin; kt < k_end; kt += SA_KT) {
+		const int j = kt + lane;
+		const bool live = j < k_end;
+		const CT *krow = Kc + (size_t)(live ? j : k_end - 1) * KL + kcol;
+		// ---- partial scores: wave w takes its slice of the key entries, every head (HP per pass)
+		for (int hp0 = 0; hp0 < Hb; hp0 += HP) {
+			const int nh = min(HP, Hb - hp0);
+			float s[HP];
+#pragma unroll
+			for (int x = 0; x < HP; ++x)
+				s[x] = 0.0f;
+			if (kvec) {
+				constexpr int U = 8; // loads in flight
+				for (int d0 = dlo; d0 < dhi; d0 += U * EPL) {
+					u32x4_t w[U];
+#pragma unroll
+					for (int u = 0; u < U; ++u)
+						w[u] = d0 + u * EPL < dhi ? load16(krow + d0 + u * EPL) : u32x4_t{0, 0, 0, 0};
+#pragma unroll
+					for (int u = 0; u < U; ++u) {
+						const int d = d0 + u * EPL;
+						if (d >= dhi)
+							break;
+						float kf[EPL];
+						if constexpr (sizeof(CT) == 2)
+							WBF16::unpack(w[u], kf);
+						else
+							WF32::unpack(w[u], kf);
+#pragma unroll
+						for (int x = 0; x < HP; ++x) {
+							if (x >= nh)
+								break;
+							const float *qp = qs + (hp0 + x) * DK8 + d;
+#pragma unroll
+							for (int e = 0; e < EPL; e += 4) {
+								const float4_t qv = *(const float4_t *)(qp + e);
+								s[x] = fmaf(qv[0], kf[e], s[x]);
+								s[x] = fmaf(qv[1], kf[e + 1], s[x]);
+								s[x] = fmaf(qv[2], kf[e + 2], s[x]);
+								s[x] = fmaf(qv[3], kf[e + 3], s[x]);
+							}
+						}
+					}
+				}
+			} else {
+				for (int d = dlo; d < dhi; ++d) {
+					float kv;
+					if constexpr (sizeof(CT) == 2)
+						kv = bf2f(krow[d]);
+					else
+						kv = krow[d];
+#pragma unroll
+					for (int x = 0; x < HP; ++x)
+						if (x < nh)
+							s[x] = fmaf(qs[(hp0 + x) * DK8 + d], kv, s[x]);
+				}
+			}
+#pragma unroll
+			for (int x = 0; x < HP; ++x)
+				if (x < nh)
+					pw[(wave * Hb + hp0 + x) * SA_KT + lane] = s[x];
+		}
+		__syncthreads();
+		// ---- running softmax, a wave per head
+		for (int r = wave; r < Hb; r += NW) {
+			float sv = 0.0f;
+#pragma unroll
+			for (int w = 0; w < NW; ++w)
+				sv += pw[(w * Hb + r) * SA_KT + lane];
+			sv = live ? sv : -FLT_MAX;
+			const float mold = mrun[r], lold = lrun[r];
+			const float mnew = fmaxf(mold, wave_max(sv));
+			const float p = live ? expf(sv - mnew) : 0.0f;
+			const float al = expf(mold - mnew);
+			const float l = lold * al + wave_sum(p);
+			ps[r * SA_KT + lane] = p;
+			if (lane == 0) {
+				mrun[r] = mnew;
+				lrun[r] = l;
+				alpha[r] = al;
+			}
+		}
+		__syncthreads();
+		// ---- weighted sums of the values
+		const int nk = min(SA_KT, k_end - kt);
+#pragma unroll
+		for (int x = 0; x < NA4; ++x) {
+			const int u = tid + x * SEQ_THREADS;
+			if (u >= Hb * V4n)
+				continue;
+			const int r = u / V4n, d4 = u % V4n;
+			const CT *vp = Vc + (size_t)kt * VL + ((h0 + r) / rep) * V + 4 * d4;
+			const float al = alpha[r];
+			float4_t v = acc[x];
+			v[0] *= al;
+			v[1] *= al;
+			v[2] *= al;
+			v[3] *= al;
+			const float *pr = ps + r * SA_KT;
+			if (vvec) {
+#pragma unroll 16
+				for (int jj = 0; jj < nk; ++jj) {
+					float c4[4];
+					if constexpr (sizeof(CT) == 2) {
+						const uint2 raw = *(const uint2 *)(vp + (size_t)jj * VL);
+						c4[0] = __builtin_bit_cast(float, raw.x << 16);
+						c4[1] = __builtin_bit_cast(float, raw.x & 0xffff0000u);
+						c4[2] = __builtin_bit_cast(float, raw.y << 16);
+						c4[3] = __builtin_bit_cast(float, raw.y & 0xffff0000u);
+					} else {
+						const float4_t raw = *(const float4_t *)(vp + (size_t)jj * VL);
+						c4[0] = raw[0];
+						c4[1] = raw[1];
+						c4[2] = raw[2];
+						c4[3] = raw[3];
+					}
+					const float p = pr[jj];
+					v[0] = fmaf(p, c4[0], v[0]);
+					v[1] = fmaf(p, c4[1], v[1]);
+					v[2] = fmaf(p, c4[2], v[2]);
+					v[3] = fmaf(p, c4[3], v[3]);
+				}
+			} else {
+				for (int jj = 0; jj < nk; ++jj) {
+					const float p = pr[jj];
+#pragma unroll
+					for (int e = 0; e < 4; ++e) {
+						if (4 * d4 + e >= V)
+							break;
+						float c;
+						if constexpr (sizeof(CT) == 2)
+							c = bf2f(vp[(size_t)jj * VL + e]);
+						else
+							c = vp[(size_t)jj * VL + e];
+						v[e] = fmaf(p, c, v[e]);
+					}
+				}
+			}
+			acc[x] = v;
+		}
+		__syncthreads(); // ps and alpha are rewritten by the next tile
+	}
+	__syncthreads();
+	const int stride = 4 * V4n + 4;
+#pragma unroll
+	for (int x = 0; x < NA4; ++x) {
+		const int u = tid + x * SEQ_THREADS;
+		if (u >= Hb * V4n)
+			continue;
+		const int r = u / V4n, d4 = u % V4n;
+		const size_t row = h0 + r;
+		if (S == 1) {
+			const float f = (gate ? gate[row] : 1.0f) / lrun[r];
+#pragma unroll
+			for (int e = 0; e < 4; ++e)
+				if (4 * d4 + e < V)
+					Ctx[row * V + 4 * d4 + e] = acc[x][e] * f;
+		} else {
+			float *pp = part + (row * S + split) * stride;
+			*(float4_t *)(pp + 4 * d4) = acc[x];
+			if (d4 == 0) {
+				pp[4 * V4n] = mrun[r];
+				pp[4 * V4n + 1] = lrun[r];
+			}
+		}
+	}
+}
+// HD = heads x dim with score mixing (the raw queries and the mixing matrix are staged), else 0
+static inline size_t sa_decode_lds_bytes(int Hb, int DK, int HD, int H) {
+	return sizeof(float) * ((size_t)Hb * ((DK + 7) & ~7) + (size_t)(1 + SEQ_THREADS / 64) * Hb * SA_KT + 3 * (size_t)Hb +
+	                        (HD ? (size_t)HD + (size_t)H * H : 0));
+}
+
 // ------------------------------------------------------------------ attention, MFMA form (portions, bf16 cache)
 // v_mfma_f32_16x16x32_bf16 products with f32 accumulation; the f32 operands (queries, softmax
 // weights) enter as hi + lo bf16 pairs (hi = bf16(x), lo = bf16(x - hi): 16 significant bits),
@@ -415,10 +737,11 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 // lane & 15). A workgroup serves one key/value head g: its 4 waves are 4 / HW blocks of 16
 // tokens x HW query heads of g (blockIdx.z: which HW heads), so one key tile and one value tile
 // in LDS feed every wave. Keys in tiles of 32 from the first key the workgroup's first token
-// sees to its last token. KS = ceil(DK / 32), NT = ceil(V / 16).
+// sees to its last token, the next tile's rows in flight (registers) during the current
+// tile's products. KS = ceil(DK / 32), NT = ceil(V / 16).
 #define SAM_KT 32
 template <int KS, int NT>
-__global__ __launch_bounds__(SEQ_THREADS) void seq_attn_mfma_kernel(const float *__restrict__ Q, int ldq, int qhs,
+__global__ __launch_bounds__(SEQ_THREADS) void seq_attn_mfma_kernel(const float *__restrict__ Q,
                                                                     const uint16_t *__restrict__ Kc,
                                                                     const uint16_t *__restrict__ Vc, AttnArgs a,
                                                                     int n_tok, int HW, const StepState *__restrict__ st,
@@ -449,14 +772,15 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_mfma_kernel(const float 
 	bf16x8_t qh[KS], ql[KS];
 	{
 		const int t = tw0 + lr;
-		const float *qrow = Q + (size_t)min(t, n_tok - 1) * ldq + (size_t)h * qhs;
+		const int tq = min(t, n_tok - 1);
 #pragma unroll
 		for (int sst = 0; sst < KS; ++sst) {
 			u32x4_t hi = {0, 0, 0, 0}, lo = {0, 0, 0, 0};
 #pragma unroll
 			for (int e = 0; e < 8; ++e) {
 				const int d = 32 * sst + 8 * lq + e;
-				const float x = (wave_on && t < n_tok && d < DK) ? qrow[d] : 0.0f;
+				const float x =
+				    (wave_on && t < n_tok && d < DK) ? attn_query(Q, tq, a.talk, a.q_mixed != 0, H, G, D, h, d) : 0.0f;
 				const uint16_t hb = f2bf(x);
 				const uint16_t lb = f2bf(x - bf2f(hb));
 				hi[e >> 1] |= (uint32_t)hb << (16 * (e & 1));
@@ -483,12 +807,18 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_mfma_kernel(const float 
 		oacc[n] = f32x4a_t{0.0f, 0.0f, 0.0f, 0.0f};
 	const bool kvec = DK % 8 == 0 && kcol % 8 == 0 && KL % 8 == 0 && (size_t)Kc % 16 == 0;
 	const bool vvec = V % 8 == 0 && VL % 8 == 0 && (size_t)Vc % 16 == 0;
-	for (int kt = klo; kt <= khi; kt += SAM_KT) {
-		__syncthreads(); // the previous tile's products have read Ks / VsT / Ps
-		for (int v = tid; v < SAM_KT * (DKP / 8); v += SEQ_THREADS) {
+	// The next tile's cache rows are fetched into registers before the current tile's products
+	// and stored to LDS after them: the global-load latency runs under the matrix work.
+	constexpr int NKL = (SAM_KT * (DKP / 8) + SEQ_THREADS - 1) / SEQ_THREADS; // 16-byte pieces per thread
+	constexpr int NVL = (SAM_KT * (VP / 8) + SEQ_THREADS - 1) / SEQ_THREADS;
+	u32x4_t kreg[NKL], vreg[NVL];
+	auto fetch = [&](int kt) {
+#pragma unroll
+		for (int i = 0; i < NKL; ++i) {
+			const int v = tid + i * SEQ_THREADS;
 			const int jj = v / (DKP / 8), d8 = (v % (DKP / 8)) * 8, j = kt + jj;
 			u32x4_t w = {0, 0, 0, 0};
-			if (j <= khi && d8 < DK) {
+			if (v < SAM_KT * (DKP / 8) && j <= khi && d8 < DK) {
 				const uint16_t *src = Kc + (size_t)j * KL + kcol + d8;
 				if (kvec && d8 + 8 <= DK) {
 					w = load16(src);
@@ -499,12 +829,14 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_mfma_kernel(const float 
 							w[e >> 1] |= (uint32_t)src[e] << (16 * (e & 1));
 				}
 			}
-			*(u32x4_t *)(Ks + jj * LDK + d8) = w;
+			kreg[i] = w;
 		}
-		for (int v = tid; v < SAM_KT * (VP / 8); v += SEQ_THREADS) {
+#pragma unroll
+		for (int i = 0; i < NVL; ++i) {
+			const int v = tid + i * SEQ_THREADS;
 			const int jj = v % SAM_KT, d8 = (v / SAM_KT) * 8, j = kt + jj;
 			u32x4_t w = {0, 0, 0, 0};
-			if (j <= khi && d8 < V) {
+			if (v < SAM_KT * (VP / 8) && j <= khi && d8 < V) {
 				const uint16_t *src = Vc + (size_t)j * VL + g * V + d8;
 				if (vvec && d8 + 8 <= V) {
 					w = load16(src);
@@ -515,10 +847,33 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_mfma_kernel(const float 
 							w[e >> 1] |= (uint32_t)src[e] << (16 * (e & 1));
 				}
 			}
-#pragma unroll
-			for (int e = 0; e < 8; ++e)
-				VsT[(d8 + e) * LDT + jj] = (uint16_t)(w[e >> 1] >> (16 * (e & 1)));
+			vreg[i] = w;
 		}
+	};
+	auto stash = [&]() {
+#pragma unroll
+		for (int i = 0; i < NKL; ++i) {
+			const int v = tid + i * SEQ_THREADS;
+			if (v < SAM_KT * (DKP / 8))
+				*(u32x4_t *)(Ks + (v / (DKP / 8)) * LDK + (v % (DKP / 8)) * 8) = kreg[i];
+		}
+#pragma unroll
+		for (int i = 0; i < NVL; ++i) {
+			const int v = tid + i * SEQ_THREADS;
+			if (v < SAM_KT * (VP / 8)) {
+				const int jj = v % SAM_KT, d8 = (v / SAM_KT) * 8;
+#pragma unroll
+				for (int e = 0; e < 8; ++e)
+					VsT[(d8 + e) * LDT + jj] = (uint16_t)(vreg[i][e >> 1] >> (16 * (e & 1)));
+			}
+		}
+	};
+	fetch(klo);
+	for (int kt = klo; kt <= khi; kt += SAM_KT) {
+		__syncthreads(); // the previous tile's products have read Ks / VsT / Ps
+		stash();
+		if (kt + SAM_KT <= khi)
+			fetch(kt + SAM_KT);
 		__syncthreads();
 		const bool need = wave_on && kt <= whi && kt + SAM_KT - 1 >= wlo;
 		if (need) {
