@@ -536,10 +536,10 @@ def layered_stack(Ly, M, width, max_tokens):
 def lenuzen_stack(Ly, M, width, max_tokens):
     """A Lenuzen-shaped stack at a real layer size: chunked attention with mixed scores and a
     sink (two layers), then sliding-window attention with biases, temperatures and output
-    gates, twice over; head size 128, four query heads per key/value head, rotary positions
+    gates, twice over; head size 128, four query heads per key/value head (at most four key/value heads), rotary positions
     on half of a head, plain feed-forwards of 3.5 x width."""
     heads = width // 128
-    kv = max(heads // 4, 1)
+    kv = min(max(heads // 4, 1), 4)  # kv_heads x dim <= 512: mixed-score portions stay on the MFMA kernel
     common = dict(heads=heads, kv_heads=kv, dim=128, vdim=128, attn_scale=128 ** -0.5, rot_dims=64, rot_base=50000.0,
                   rot_factor=4.0, rot_orig=4096, rot_fast=32.0, rot_slow=1.0, ff_kind=Ly.FF_PLAIN, ff=width * 7 // 2)
     chunked = dict(mask_kind=Ly.MASK_CHUNK, mask_size=2048, qk_norm=Ly.QK_WHOLE, sink=1, talking=True, **common)

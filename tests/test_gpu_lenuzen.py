@@ -398,6 +398,61 @@ def test_greedy_graph_replays_match_eager_steps(rt):
         model.close()
 
 
+_LONG_REF = {}
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_prompt_longer_than_one_internal_portion(rt, dtype):
+    """A step of more tokens than the engine's work buffers hold (4096) is cut inside the
+    engine, in the middle of a window and of a chunk; asked rows on both sides of the cut
+    come back in order."""
+    cfg = C.config([("attention", C.window(heads=2, kv_heads=1, dim=8, vdim=8, size=150, rot_dims=4, scale=0.35), None),
+                    ("attention_2", C.chunk(heads=2, kv_heads=2, dim=8, vdim=8, size=1000, rot_dims=8, scale=0.35), None)],
+                   width=32, vocab=53)
+    model, dec, w = build(rt, cfg, wdt_of(dtype), seed=16, max_tokens=4300)
+    try:
+        tok = C.tokens(cfg, 4200, 15)
+        want = [0, 5, 3999, 4000, 4094, 4095, 4096, 4097, 4150, 4199]
+        got = dec.step(tok, want)
+        assert dec.pos == len(tok)
+        if "ref" not in _LONG_REF:  # the same weights and tokens for both matrix types
+            _LONG_REF["ref"] = R.forward(cfg, w, tok)[want]
+        assert rel_err(got, _LONG_REF["ref"]).max() < tol(dtype)
+    finally:
+        dec.close()
+        model.close()
+
+
+def test_sequence_cannot_pass_max_tokens(rt):
+    from yalm_amd import models as M
+
+    model, dec, _ = build(rt, C.ONLY_WINDOW, M.F32, seed=13, max_tokens=16)
+    try:
+        dec.step(C.tokens(C.ONLY_WINDOW, 16, 0))
+        with pytest.raises(rt.YalmError):
+            dec.step([1])
+    finally:
+        dec.close()
+        model.close()
+
+
+def test_mixed_scores_over_a_long_key_row(rt):
+    """kv_heads x dim above the MFMA attention's key size: portions of a bf16 model take the
+    f32 FMA kernel, with the same results."""
+    from yalm_amd import models as M
+
+    cfg = C.config([("attention_2", C.chunk(heads=10, kv_heads=5, dim=128, vdim=8, size=50, rot_dims=64, scale=0.09), None)],
+                   width=64, vocab=101)
+    model, dec, w = build(rt, cfg, M.BF16, seed=18)
+    try:
+        tok = C.tokens(cfg, 120, 17)
+        ref = R.forward(cfg, w, tok)
+        assert rel_err(run_portions(dec, tok, [70, 3, 1, 1]), ref).max() < BF16_TOL
+    finally:
+        dec.close()
+        model.close()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_runner(rt, tmp_path, dtype):
     """bin/trace_run on a checkpoint folder written here: two requests one after the other,

@@ -673,7 +673,7 @@ static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q,
 		if (ks <= 8) return attn_mfma_launch<8>(q, li, n, a, Q, gate, ctx);
 		return attn_mfma_launch<16>(q, li, n, a, Q, gate, ctx);
 	}
-	const int Hb = talk ? a.H : a.H / a.G, Gb = talk ? a.G : 1, V4n = (a.V + 3) / 4, D4 = (a.D + 3) & ~3;
+	const int Hb = a.H / a.G, Gb = talk ? a.G : 1, V4n = (a.V + 3) / 4, D4 = (a.D + 3) & ~3;
 	const CT *Kc = (const CT *)q->cache[li], *Vc = (const CT *)q->vcache[li];
 	const int rep = a.H / a.G;
 	const size_t dec_lds = sa_decode_lds_bytes(rep, DK, talk ? a.H * a.D : 0, a.H);
@@ -710,8 +710,12 @@ static int attn_core_t(Seq *q, int li, int n, const AttnArgs &a, const float *Q,
 		--TQ;
 	const int R = TQ * Hb;
 	const int S = n <= GEMV_MAX_M ? q->attn_splits[li] : 1;
-	const dim3 g(cdiv(n, TQ), S, talk ? 1 : a.G);
+	const dim3 g(cdiv(n, TQ), S, a.G);
 	const size_t lds = sa_lds_bytes(R, Gb, a.D, a.V);
+	if (lds > 160 * 1024 - 64) {
+		set_err("attention: one token's queries of a key/value head's heads over the whole key row do not fit in LDS");
+		return YALM_ERR_UNSUPPORTED;
+	}
 	const int na = cdiv(R * V4n, SEQ_THREADS);
 #define SA_LAUNCH(NA)                                                                                                  \
 	do {                                                                                                               \

@@ -233,12 +233,12 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_prep_kernel(const float 
 }
 
 // ------------------------------------------------------------------ attention, f32 FMA form
-// A workgroup owns TQ tokens x Hb heads (rows r = tq Hb + hl) and walks its share of the keys
-// they see in tiles of SA_KT. Without score mixing the heads are those of one key/value head
-// (gridDim.z = G, key columns of that head); with it, all heads, whose (mixed) queries span
+// A workgroup owns TQ tokens x the Hb = H / G heads of one key/value head (gridDim.z = G; rows
+// r = tq Hb + hl) and walks its share of the keys they see in tiles of SA_KT. Without score
+// mixing the keys are that head's columns of the cache rows; with it the (mixed) queries span
 // the whole key row, taken in G column chunks of D that accumulate into the same scores. Per
 // tile: scores of every row (a lane per key), mask and running softmax per row, then the
-// weighted sums of the value tile(s), each thread NA4 groups of 4 value entries of one row.
+// weighted sums of the value tile, each thread NA4 groups of 4 value entries of one row.
 // Key splits (gridDim.y = S > 1; single tokens and short portions): split s leaves (sums,
 // running maximum, running sum) per row in `part` for seq_latent_merge_kernel; the sink (a key
 // of score 0 without a value) is split 0's starting state. S == 1 writes the normalised,
@@ -307,8 +307,8 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 	extern __shared__ __attribute__((aligned(16))) float lds[];
 	const int H = a.H, G = a.G, D = a.D, V = a.V, rep = H / G;
 	const bool talk = a.talk != nullptr;
-	const int Hb = talk ? H : rep, Gb = talk ? G : 1;
-	const int h0 = talk ? 0 : blockIdx.z * rep, g0 = talk ? 0 : blockIdx.z;
+	const int Hb = rep, Gb = talk ? G : 1;
+	const int h0 = blockIdx.z * rep, g0 = talk ? 0 : blockIdx.z, vg = blockIdx.z;
 	const int R = TQ * Hb;
 	const int D4 = (D + 3) & ~3, q4n = D4 >> 2, V4n = (V + 3) >> 2, ldk = sa_ldk(D, V), ldqs = Gb * D4;
 	float *qs = lds;                  // [R][Gb][D4]
@@ -413,9 +413,9 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 			}
 		}
 		// ---- weighted sums of the values
-		for (int gl = 0; gl < Gb; ++gl) {
+		{
 			__syncthreads(); // the weights are written / the previous readers of cs are done
-			sa_fill_tile<CT>(cs, ldk, Vc, G * V, (g0 + gl) * V, V, kt, k_end);
+			sa_fill_tile<CT>(cs, ldk, Vc, G * V, vg * V, V, kt, k_end);
 			__syncthreads();
 #pragma unroll
 			for (int x = 0; x < NA4; ++x) {
@@ -423,8 +423,6 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_attn_kernel(const float *__re
 				if (u >= R * V4n)
 					continue;
 				const int r = u / V4n, d4 = u % V4n;
-				if ((h0 + r % Hb) / rep != g0 + gl)
-					continue;
 				const float al = alpha[r];
 				float4_t v = acc[x];
 				v[0] *= al;
