@@ -168,3 +168,24 @@ def test_lenuzen_restatement_is_causal_and_masks_hold():
     assert m[5, 4] and not m[4, 3] and m[7, 4] and not m[8, 7] and not m[3, 4]
     p = LR.softmax_rows(np.zeros((1, 3)), np.array([[True, True, False]]), True)
     assert np.allclose(p, [[1 / 3, 1 / 3, 0.0]])
+
+
+def test_bench_stacks_are_valid_layer_list_configurations():
+    """The stacks bench.py --layered times: every layer's packed tensor set is well formed at
+    every benchmarked width, and mixed-score layers keep their key row within the MFMA
+    attention kernel's key size."""
+    import bench
+
+    for width in (1024, 2048, 4096):
+        for make in (bench.layered_stack, bench.lenuzen_stack):
+            c = make(Ly, M, width, 2112)
+            assert c.width == width and len(c.layers) == 6
+            for l in c.layers:
+                shapes = Ly.packed_shapes(c, l)
+                assert shapes["w_in"][0] == (l.in_rows, width) and shapes["w_o"][0] == (width, l.mix_out)
+                if l.mixer == Ly.MIX_ATTN:
+                    assert l.heads % l.kv_heads == 0 and l.rot_dims <= l.dim
+                    if l.talking:
+                        assert l.kv_heads * l.dim <= 512 and "talk" in shapes
+    c = bench.lenuzen_stack(Ly, M, 2048, 2112)
+    assert (c.norm_kind, c.pre_norm, c.pos_embed, c.tied_head) == (Ly.NORM_LAYER, False, False, True)
