@@ -398,6 +398,58 @@ def test_greedy_graph_replays_match_eager_steps(rt):
         model.close()
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_attention_options_combine_freely(rt, dtype):
+    """The attention mixer's options are parameters of the engine, not of one design: a layer
+    put together by hand (full causal mask, no query / key norm, unit-rms values, a sink, head
+    temperatures, rotation over the whole head without rescaling, no gate, no mixing) inside
+    the other envelope (rms norms, an opening norm per sublayer, an untied head) against the
+    same combination restated from the per-mechanism functions."""
+    from yalm_amd import layered as Ly
+
+    W, V_, H, G, D, Vd, T = 48, 67, 4, 2, 16, 24, 90
+    rng = np.random.default_rng(5)
+
+    def rnd(*shape, s=None):
+        a = rng.standard_normal(shape) * (s if s is not None else 1.0 / np.sqrt(shape[-1]))
+        return Ly.bf16_to_f32(Ly.f32_to_bf16(a.astype(np.float32))).reshape(shape)
+
+    t = {"embed": rnd(V_, W, s=0.1), "head": rnd(V_, W), "q": rnd(H * D, W), "k": rnd(G * D, W), "v": rnd(G * Vd, W),
+         "o": rnd(W, H * Vd), "norm1": 1 + rnd(W, s=0.2), "norm1b": 1 + rnd(W, s=0.2), "final": 1 + rnd(W, s=0.2),
+         "temp": np.float32(1.0) + np.abs(rnd(H, s=0.5))}
+    spec = Ly.LayerSpec(Ly.MIX_ATTN, heads=H, kv_heads=G, dim=D, vdim=Vd, attn_scale=0.8, mask_kind=Ly.MASK_CAUSAL,
+                        qk_norm=Ly.QK_NONE, v_norm=1, sink=1, rot_dims=D, rot_base=100.0, head_temps=True)
+    c = Ly.LayeredConfig("by hand", W, V_, [spec], embed_scale=3.0, norm_eps=1e-5, max_tokens=128, weight_dtype=wdt_of(dtype),
+                         norm_kind=Ly.NORM_RMS, pre_norm=True, pos_embed=False, logit_scale=1.25)
+    as_w = (lambda a: np.ascontiguousarray(a, np.float32)) if dtype == "f32" else Ly.f32_to_bf16
+    layer = {"norm1": t["norm1"], "norm1b": t["norm1b"], "w_in": as_w(np.concatenate([t["q"], t["k"], t["v"]])),
+             "w_o": as_w(t["o"]), "head_temp": t["temp"]}
+    assert set(layer) == set(Ly.packed_shapes(c, spec))
+    model = rt.SeqModel.from_packed(c, {"embed": as_w(t["embed"]), "final_norm": t["final"], "head": as_w(t["head"]),
+                                        "layers": [layer]})
+    dec = rt.SeqDecoder(model)
+    try:
+        w = {k: v.astype(np.float64) for k, v in t.items()}
+        tok = rng.integers(0, V_, T).tolist()
+        eps = 1e-5
+        x = w["embed"][tok] * 3.0
+        h = R.unit_rms(x, eps) * w["norm1"]
+        rot = {"dims": D, "base": 100.0}
+        pos = np.arange(T)
+        q = R.rotate((h @ w["q"].T).reshape(T, H, D), rot, pos)
+        k = R.rotate((h @ w["k"].T).reshape(T, G, D), rot, pos)
+        v = R.unit_rms((h @ w["v"].T).reshape(T, G, Vd), eps)
+        o, _ = R.attention_core(q, k, v, 0.8, R.visible("causal", 0, T), temp=w["temp"], sink=True)
+        x = x + R.unit_rms(o.reshape(T, H * Vd) @ w["o"].T, eps) * w["norm1b"]
+        ref = (R.unit_rms(x, eps) * w["final"]) @ w["head"].T * 1.25
+        assert rel_err(dec.step(tok, list(range(T))), ref).max() < tol(dtype)
+        dec.reset()
+        assert rel_err(run_portions(dec, tok, [40, 2, 9] + [1] * 39), ref).max() < tol(dtype)
+    finally:
+        dec.close()
+        model.close()
+
+
 _LONG_REF = {}
 
 
