@@ -44,6 +44,8 @@ struct yalm_seq_s {
 	int zw = 0;                  // floats per row of Z (the widest input projection)
 	float *X = nullptr, *Hn = nullptr, *Y = nullptr, *Z = nullptr, *B[4] = {};
 	const float *In = nullptr;   // what a sublayer reads: Hn (pre_norm) or X itself
+	float *Xalt = nullptr, *Xbase = nullptr; // single tokens without opening norms: the stream alternates between two rows
+	const float *pend_wb = nullptr; // a closing norm not yet applied: X += norm(Y) pend_wb, owed to the next product
 	bool ln = false;             // the model's norms are layer norms
 	float *inv_freq = nullptr;
 	uint16_t *a16 = nullptr;     // [cap][bw] bf16 copy of a product's activations (large-tile GEMM operand)
@@ -338,6 +340,9 @@ static int create_seq(const yalm_seq_config *config, const yalm_seq_weights *w, 
 	STRY(sallocT(q, &q->gen_tokens, q->gen_cap));
 	q->ln = c.norm_kind == YALM_NORM_LAYER;
 	q->In = c.pre_norm ? q->Hn : q->X;
+	q->Xbase = q->X;
+	if (!c.pre_norm)
+		STRY(sallocT(q, &q->Xalt, (size_t)c.width));
 	// position frequencies 10000^(-2 i / width), evaluated in double
 	if (c.pos_embed) {
 		std::vector<float> f((c.width + 1) / 2);
@@ -646,6 +651,51 @@ static int mixer_delta(Seq *q, int li, int n) {
 	return gemm(q, plain(on, CV, l.w_o, CV, q->Y, c.width, n, c.width, CV));
 }
 
+// ---- the closing norm of a single token, owed to the product that reads the stream next
+static int add_norm(Seq *q, const float *wb, const float *w_next, int n, const yalm_seq_layer *moe);
+
+static bool an_foldable(const Seq *q, int n) {
+	return n == 1 && !q->c.pre_norm && !q->dump_on && q->Xalt && q->c.width % 8 == 0 && q->c.width <= 8 * 1024;
+}
+static int flush_norm(Seq *q, int n) {
+	if (!q->pend_wb)
+		return YALM_OK;
+	const float *wb = q->pend_wb;
+	q->pend_wb = nullptr;
+	return add_norm(q, wb, nullptr, n, nullptr);
+}
+template <class WT>
+static int gemv_an_t(Seq *q, const GemmArgs &a) {
+	const int K = a.K, ki = cdiv(K, 1024);
+	const dim3 g(cdiv(a.N, (SEQ_THREADS / 64) * GAN_RPW));
+#define GA_LAUNCH(KI)                                                                                                  \
+	seq_gemv_an_kernel<WT, KI><<<g, SEQ_THREADS, (size_t)K * sizeof(float), q->stream>>>(                              \
+	    q->X, q->Y, q->pend_wb, q->c.norm_eps, (int)q->ln, K, q->X == q->Xbase ? q->Xalt : q->Xbase, a.W, a.N, a.C,    \
+	    a.bias, a.epi)
+	if (ki <= 1) GA_LAUNCH(1);
+	else if (ki <= 2) GA_LAUNCH(2);
+	else if (ki <= 4) GA_LAUNCH(4);
+	else GA_LAUNCH(8);
+#undef GA_LAUNCH
+	HIPCHK(hipGetLastError());
+	q->X = q->X == q->Xbase ? q->Xalt : q->Xbase; // the stream now lives in the other row
+	q->In = q->X;
+	q->pend_wb = nullptr;
+	return YALM_OK;
+}
+// A product whose A operand is the sublayer input q->In. With a closing norm owed and a single
+// token, the norm + residual sum run inside the product's kernel; else the norm first.
+static int gemm_in(Seq *q, GemmArgs a) {
+	if (q->pend_wb) {
+		if (a.M == 1 && !a.W2 && (a.epi == EPI_NONE || a.epi == EPI_GELU) && a.ldw == a.K && a.K == q->c.width &&
+		    (size_t)a.W % 16 == 0 && !a.rows && !a.w_sel && a.z_split == 0 && a.A == q->In)
+			return q->c.weight_dtype == YALM_F32 ? gemv_an_t<WF32>(q, a) : gemv_an_t<WBF16>(q, a);
+		TRY(flush_norm(q, a.M));
+		a.A = q->In;
+	}
+	return gemm(q, a);
+}
+
 template <int KS>
 static int attn_mfma_launch(Seq *q, int li, int n, const AttnArgs &a, const float *Q, const float *gate, float *ctx) {
 	const int rep = a.H / a.G, HW = rep >= 4 ? 4 : (rep >= 2 ? 2 : 1), NT = cdiv(a.V, 16);
@@ -752,7 +802,7 @@ static int mixer_attn(Seq *q, int li, int n) {
 	{
 		GemmArgs g = plain(q->In, c.width, l.w_in, c.width, q->Z, zin, n, zmain, c.width);
 		g.bias = l.in_bias;
-		TRY(gemm(q, g));
+		TRY(gemm_in(q, g));
 	}
 	AttnArgs a;
 	a.H = H;
@@ -801,7 +851,7 @@ static int ff_plain(Seq *q, int li, int n) {
 	const yalm_seq_config &c = q->c;
 	GemmArgs a = plain(q->In, c.width, l.w_up, c.width, q->B[0], l.ff, n, l.ff, c.width);
 	a.epi = EPI_GELU;
-	TRY(gemm(q, a));
+	TRY(gemm_in(q, a));
 	return gemm(q, plain(q->B[0], l.ff, l.w_down, l.ff, q->Y, c.width, n, c.width, l.ff));
 }
 
@@ -876,7 +926,7 @@ static int ff_moe(Seq *q, int li, int n) {
 }
 
 // moe: the layer's routed experts feed the norm (their combine happens inside it) instead of Y
-static int add_norm(Seq *q, const float *wb, const float *w_next, int n, const yalm_seq_layer *moe = nullptr) {
+static int add_norm(Seq *q, const float *wb, const float *w_next, int n, const yalm_seq_layer *moe) {
 	const int w = q->c.width;
 	if (!moe && w <= 16 * SEQ_THREADS) { // the row in registers
 #define AN_LAUNCH(E)                                                                                                   \
@@ -901,6 +951,20 @@ static int enqueue_portion(Seq *q, const int *tokens_dev, int n) {
 	const yalm_seq_config &c = q->c;
 	const bool pre = c.pre_norm != 0; // else the sublayers read the stream itself and no opening norm is computed
 	const float *first_norm = pre ? q->L[0].norm1 : nullptr;
+	if (!pre) { // every portion starts in the same row of the stream (the greedy graph's pointers are static)
+		q->X = q->Xbase;
+		q->In = q->X;
+	}
+	q->pend_wb = nullptr;
+	const bool fold = an_foldable(q, n);
+	// the closing norm of a sublayer: applied now, or owed to the product that reads the stream next
+	auto close = [&](const float *wb, const float *w_next, const yalm_seq_layer *moe) {
+		if (fold && !moe && !w_next) {
+			q->pend_wb = wb;
+			return (int)YALM_OK;
+		}
+		return add_norm(q, wb, w_next, n, moe);
+	};
 	if (c.weight_dtype == YALM_F32)
 		seq_embed_kernel<WF32><<<n, SEQ_THREADS, 0, q->stream>>>(q->st, tokens_dev, q->embed, q->inv_freq, c.width,
 		                                                         c.vocab, c.embed_scale, q->X, first_norm, c.norm_eps,
@@ -913,6 +977,8 @@ static int enqueue_portion(Seq *q, const int *tokens_dev, int n) {
 	for (int li = 0; li < c.n_layers; ++li) {
 		const yalm_seq_layer &l = q->L[li];
 		const float *next = pre && li + 1 < c.n_layers ? q->L[li + 1].norm1 : nullptr;
+		if (l.mixer != YALM_MIX_ATTN)
+			TRY(flush_norm(q, n)); // only the attention mixer's input projection takes an owed norm
 		if (l.mixer == YALM_MIX_LATENT)
 			TRY(mixer_latent(q, li, n));
 		else if (l.mixer == YALM_MIX_RGLRU)
@@ -922,18 +988,20 @@ static int enqueue_portion(Seq *q, const int *tokens_dev, int n) {
 		else
 			TRY(mixer_delta(q, li, n));
 		if (l.ff_kind == YALM_FF_NONE) {
-			TRY(add_norm(q, l.norm1b, next, n));
+			TRY(close(l.norm1b, next, nullptr));
 		} else {
-			TRY(add_norm(q, l.norm1b, pre ? l.norm2 : nullptr, n));
+			TRY(close(l.norm1b, pre ? l.norm2 : nullptr, nullptr));
+			if (l.ff_kind != YALM_FF_PLAIN)
+				TRY(flush_norm(q, n));
 			TRY(l.ff_kind == YALM_FF_DENSE ? ff_dense(q, li, n)
 			                               : (l.ff_kind == YALM_FF_PLAIN ? ff_plain(q, li, n) : ff_moe(q, li, n)));
-			TRY(add_norm(q, l.norm2b, next, n, l.ff_kind == YALM_FF_MOE ? &l : nullptr));
+			TRY(close(l.norm2b, next, l.ff_kind == YALM_FF_MOE ? &l : nullptr));
 		}
 		if (q->dump_on && q->dump)
 			HIPCHK(hipMemcpyAsync(q->dump + (size_t)li * n * c.width, q->X, (size_t)n * c.width * sizeof(float),
 			                      hipMemcpyDeviceToDevice, q->stream));
 	}
-	return YALM_OK;
+	return flush_norm(q, n); // the last sublayer's norm, if still owed
 }
 
 // Final norm of the asked rows and their logits into q->logits ([n_rows][vocab], n_rows <= LOGIT_ROWS).

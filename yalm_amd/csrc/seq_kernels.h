@@ -531,6 +531,111 @@ __global__ __launch_bounds__(SEQ_THREADS) void seq_gemv_kernel(GemmArgs a) {
 	}
 }
 
+// ---- one token, the previous sublayer's closing norm folded in: x' = x + norm(y) wb is what
+// the product reads when sublayers read the stream itself. Every workgroup rebuilds x' once
+// (a thread KI groups of 4 entries, the row's statistics over the workgroup) into LDS, while
+// its waves' first weight rows are already in flight; then each wave multiplies RPW weight
+// rows: C[n] = epi(W[n] . x' + bias[n]). Workgroup 0 also writes x' to Xout, a second buffer
+// (the other workgroups still read X). K % 8 == 0, K <= 1024 KI, rows of W contiguous and
+// 16-byte aligned. Dynamic LDS: K floats.
+#define GAN_RPW 2
+template <class WT, int KI>
+__global__ __launch_bounds__(SEQ_THREADS) void seq_gemv_an_kernel(const float *__restrict__ X, const float *__restrict__ Y,
+                                                                  const float *__restrict__ wb, float eps, int ln, int K,
+                                                                  float *__restrict__ Xout, const void *__restrict__ W,
+                                                                  int N, float *__restrict__ C,
+                                                                  const float *__restrict__ bias, int epi) {
+	extern __shared__ __attribute__((aligned(16))) float xs[];
+	__shared__ float red[SEQ_THREADS / 64];
+	constexpr int KE = 2 * KI;                 // steps of 512 entries over a weight row
+	constexpr int NL = WT::BYTES == 2 ? 1 : 2; // 16-byte loads per 8 weights
+	const int tid = threadIdx.x, lane = tid & 63;
+	const int n0 = (blockIdx.x * (SEQ_THREADS / 64) + (tid >> 6)) * GAN_RPW;
+	u32x4_t wv[KE][NL];
+	auto fetch = [&](int n) {
+		const char *w = (const char *)W + (size_t)n * K * WT::BYTES;
+#pragma unroll
+		for (int u = 0; u < KE; ++u) {
+			const int k = u * 512 + lane * 8;
+#pragma unroll
+			for (int i = 0; i < NL; ++i)
+				wv[u][i] = (n < N && k < K) ? load_nt16(w + (size_t)k * WT::BYTES + 16 * i) : u32x4_t{0, 0, 0, 0};
+		}
+	};
+	fetch(n0);
+	float4_t x[KI], y[KI], b[KI];
+	float sm = 0.0f;
+#pragma unroll
+	for (int i = 0; i < KI; ++i) {
+		const int k = 4 * (tid + SEQ_THREADS * i);
+		const bool in = k < K;
+		y[i] = in ? *(const float4_t *)(Y + k) : float4_t{0, 0, 0, 0};
+		x[i] = in ? *(const float4_t *)(X + k) : float4_t{0, 0, 0, 0};
+		b[i] = in ? *(const float4_t *)(wb + k) : float4_t{0, 0, 0, 0};
+		sm += (y[i][0] + y[i][1]) + (y[i][2] + y[i][3]);
+	}
+	if (ln) { // entries past the row's end stay 0
+		const float mu = block_sum(sm, red) / (float)K;
+#pragma unroll
+		for (int i = 0; i < KI; ++i)
+			if (4 * (tid + SEQ_THREADS * i) < K)
+#pragma unroll
+				for (int e = 0; e < 4; ++e)
+					y[i][e] -= mu;
+	}
+	float ss = 0.0f;
+#pragma unroll
+	for (int i = 0; i < KI; ++i)
+#pragma unroll
+		for (int e = 0; e < 4; ++e)
+			ss = fmaf(y[i][e], y[i][e], ss);
+	const float r = 1.0f / sqrtf(block_sum(ss, red) / (float)K + eps);
+#pragma unroll
+	for (int i = 0; i < KI; ++i) {
+		const int k = 4 * (tid + SEQ_THREADS * i);
+		if (k >= K)
+			continue;
+#pragma unroll
+		for (int e = 0; e < 4; ++e)
+			x[i][e] = fmaf(y[i][e] * r, b[i][e], x[i][e]);
+		*(float4_t *)(xs + k) = x[i];
+		if (blockIdx.x == 0)
+			*(float4_t *)(Xout + k) = x[i];
+	}
+	__syncthreads();
+#pragma unroll
+	for (int j = 0; j < GAN_RPW; ++j) {
+		const int n = n0 + j;
+		float acc = 0.0f;
+#pragma unroll
+		for (int u = 0; u < KE; ++u) {
+			const int k = u * 512 + lane * 8;
+			if (k >= K)
+				continue;
+			float wf[8];
+			if constexpr (WT::BYTES == 2) {
+				WT::unpack(wv[u][0], wf);
+			} else {
+				WT::unpack(wv[u][0], wf);
+				WT::unpack(wv[u][NL - 1], wf + 4);
+			}
+			const float4_t x0 = *(const float4_t *)(xs + k), x1 = *(const float4_t *)(xs + k + 4);
+#pragma unroll
+			for (int e = 0; e < 4; ++e) {
+				acc = fmaf(wf[e], x0[e], acc);
+				acc = fmaf(wf[4 + e], x1[e], acc);
+			}
+		}
+		if (j + 1 < GAN_RPW)
+			fetch(n + 1); // the next row's loads run under this row's reduction
+		acc = wave_sum(acc);
+		if (lane == 0 && n < N) {
+			const float v = acc + (bias ? bias[n] : 0.0f);
+			C[n] = epi == EPI_GELU ? sq_gelu_tanh(v) : v;
+		}
+	}
+}
+
 // ---- portions: 64 x 64 output tiles, K in slabs of 32 through LDS.
 #define GT_BM 64
 #define GT_BN 64
