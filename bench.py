@@ -540,15 +540,15 @@ def lenuzen_stack(Ly, M, width, max_tokens):
     on half of a head, plain feed-forwards of 3.5 x width."""
     heads = width // 128
     kv = min(max(heads // 4, 1), 4)  # kv_heads x dim <= 512: mixed-score portions stay on the MFMA kernel
-    common = dict(heads=heads, kv_heads=kv, dim=128, vdim=128, attn_scale=128 ** -0.5, rot_dims=64, rot_base=50000.0,
-                  rot_factor=4.0, rot_orig=4096, rot_fast=32.0, rot_slow=1.0, ff_kind=Ly.FF_PLAIN, ff=width * 7 // 2)
+    common = dict(heads=heads, kv_heads=kv, dim=128, vdim=128, attn_scale=128 ** -0.5, rot_dims=64, rot_base=500000.0,
+                  rot_factor=8.0, rot_orig=8192, rot_fast=16.0, rot_slow=2.0, ff_kind=Ly.FF_PLAIN, ff=width * 7 // 2)
     chunked = dict(mask_kind=Ly.MASK_CHUNK, mask_size=2048, qk_norm=Ly.QK_WHOLE, sink=1, talking=True, **common)
     windowed = dict(mask_kind=Ly.MASK_WINDOW, mask_size=1024, qk_norm=Ly.QK_HEAD_UNIT, v_norm=1, out_gate=1,
                     in_biased=True, head_temps=True, **common)
     layers = [Ly.LayerSpec(Ly.MIX_ATTN, **d) for d in (chunked, chunked, windowed, chunked, chunked, windowed)]
-    return Ly.LayeredConfig("Lenuzen", width, 32000, layers, embed_scale=1.0, norm_eps=1e-6, max_tokens=max_tokens,
+    return Ly.LayeredConfig("Lenuzen", width, 32000, layers, embed_scale=1.0, norm_eps=1e-5, max_tokens=max_tokens,
                             weight_dtype=M.BF16, norm_kind=Ly.NORM_LAYER, pre_norm=False, pos_embed=False,
-                            logit_scale=0.5, tied_head=True)
+                            logit_scale=0.7, tied_head=True)
 
 
 def layered_bench(args, out_file):
